@@ -1,0 +1,384 @@
+"""Benchmark of the quantized-linear forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5] [--m M]
+
+Default workload: BASELINE.json configs[1] - the DiT-XL/2 MLP pair, W4A4, bf16,
+M = 2048 tokens: fc1 1152->4608, GELU, fc2 4608->1152.  One step = rotate+quantize,
+packed GEMM, GELU, rotate+quantize, packed GEMM, with the input already resident
+in HBM.  Prints ONE JSON line; `value` is whole-step TFLOP/s counted as 2*M*N*K
+per linear.  The `roofline` object is for the dominant kernel (the packed GEMM,
+or the streaming kernel for the small-M workload c5), timed alone with events on
+the launch stream.  `cpu_baseline` times the CPU oracle (a port of the
+reference's CPU path) on a bounded row sample of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--m", type=int, default=0, help="token count override (c5: 1, 4 or 16)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-iters", type=int, default=50)
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------- workloads
+
+def workload_spec(name: str, m_override: int):
+    """-> dict(name, M, dtype, layers=[(K, N, wbits, abits, block, act_after)], x_kind)"""
+    if name == "c1":
+        return dict(name="c1 single W4A4 linear 1152->1152, fp32, block 64", M=m_override or 256,
+                    dtype=torch.float32, x_kind="entry_outliers",
+                    layers=[(1152, 1152, 4, 4, 64, None)], w_std=0.02)
+    if name == "c2":
+        return dict(name="c2 DiT-XL/2 MLP pair W4A4 bf16 (1152->4608, GELU, 4608->1152)", M=m_override or 2048,
+                    dtype=torch.bfloat16, x_kind="column_outliers",
+                    layers=[(1152, 4608, 4, 4, "paper", "gelu"), (4608, 1152, 4, 4, "paper", None)], w_std=0.02)
+    if name == "c3":
+        return dict(name="c3 Flux double-stream projections W3A3 bf16 (qkv, out, fc1, fc2)", M=m_override or 4608,
+                    dtype=torch.bfloat16, x_kind="student_t",
+                    layers=[(3072, 9216, 3, 3, "paper", "slice3072"), (3072, 3072, 3, 3, "paper", None),
+                            (3072, 12288, 3, 3, "paper", "gelu"), (12288, 3072, 3, 3, "paper", None)], w_std=0.02)
+    if name == "c4":
+        return dict(name="c4 video-DiT FFN W4A6 bf16 (5120->13824, GELU, 13824->5120)", M=m_override or 32760,
+                    dtype=torch.bfloat16, x_kind="entry_outliers",
+                    layers=[(5120, 13824, 4, 6, "paper", "gelu"), (13824, 5120, 4, 6, "paper", None)], w_std=0.015)
+    # c5: one interior layer group of the 40-layer decode stack (q,k W2; v,o W3; MLP W3) is
+    # built per distinct matrix; see build_c5
+    return dict(name="c5 small-M decode stack, mixed W2/W3/W4, A4", M=m_override or 1, dtype=torch.bfloat16,
+                x_kind="plain", layers=[], w_std=0.02)
+
+
+def make_input(spec, k, gen):
+    m = spec["M"]
+    x = torch.randn(m, k, generator=gen)
+    kind = spec["x_kind"]
+    if kind == "entry_outliers":
+        mask = torch.rand(m, k, generator=gen) < 0.01
+        x = torch.where(mask, x * 20, x)
+    elif kind == "column_outliers":
+        cols = torch.randperm(k, generator=gen)[: max(1, int(np.ceil(0.005 * k)))]
+        x[:, cols] *= 30
+    elif kind == "student_t":
+        chi = torch.randn(m, k, 4, generator=gen).square().sum(-1)
+        x = x / torch.sqrt(chi / 4)
+    return x.to(spec["dtype"])
+
+
+def random_packed_weight(n, k, bits, gen, device):
+    """Synthetic quantized weight: uniform random indices (the matmul kernels do not care
+    how indices were chosen) and row norms of N(0, std) rows."""
+    nbytes = (n * k * bits + 7) // 8
+    packed = torch.randint(0, 256, (nbytes,), generator=gen, dtype=torch.uint8)
+    return packed.to(device)
+
+
+def build_layers(spec, device, gen, real_quantization: bool):
+    from orbitquant_amd import OrbitLinear, OrbitQuantConfig
+
+    layers = []
+    for (k, n, wbits, abits, block, act) in spec["layers"]:
+        cfg = OrbitQuantConfig(weight_bits=wbits, activation_bits=abits, block_size=block)
+        if real_quantization:
+            w = torch.randn(n, k, generator=gen) * spec["w_std"]
+            layer = OrbitLinear.from_weight(w, bias=torch.zeros(n), config=cfg)
+        else:
+            packed = torch.randint(0, 256, ((n * k * wbits + 7) // 8,), generator=gen, dtype=torch.uint8)
+            norms = (torch.full((n,), spec["w_std"] * np.sqrt(k)) * (1 + 0.05 * torch.randn(n, generator=gen))).to(torch.bfloat16)
+            layer = OrbitLinear(in_features=k, out_features=n, config=cfg, bias=torch.zeros(n),
+                                packed_weight_indices=packed, row_norms=norms)
+        layer = layer.to(device)
+        if layer.bias is not None:
+            layer.bias.data = layer.bias.data.to(spec["dtype"])
+        layers.append((layer, act))
+    return layers
+
+
+def run_step(layers, x):
+    h = x
+    for layer, act in layers:
+        h = layer(h)
+        if act == "gelu":
+            h = torch.nn.functional.gelu(h)
+        elif act == "slice3072":
+            h = h[..., :3072].contiguous()
+    return h
+
+
+# ------------------------------------------------------------ kernel-only timing
+
+def time_kernel(fn, iters):
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters * 1e-3  # seconds per launch
+
+
+def gemm_only_closure(layer, x):
+    """The matmul launch of `layer` alone, on pre-computed activation codes."""
+    from orbitquant_amd import ops
+
+    k = layer.in_features
+    if layer.activation_bits <= 4:
+        codes, _, norms = ops.rotate_quantize(
+            x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
+            block_size=layer.rotation.block_size, eps=layer.activation_eps,
+            inv_sqrt_block=layer.rotation.normalization, code_format="nibble")
+        bias = layer.bias
+
+        def fn():
+            return ops.packed_linear(
+                codes, norms, layer._activation_codebook_centroids, layer.packed_weight_indices, layer.row_norms,
+                layer._weight_codebook_centroids, code_format="nibble", activation_bits=layer.activation_bits,
+                weight_bits=layer.weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
+                output_dtype=x.dtype)
+        return fn
+    _, unit, norms = ops.rotate_quantize(
+        x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
+        block_size=layer.rotation.block_size, eps=layer.activation_eps,
+        inv_sqrt_block=layer.rotation.normalization, centroids=layer._activation_codebook_centroids,
+        code_format=None, values="unit_bf16")
+    flat_norms = norms.reshape(-1)
+
+    def fn():
+        return ops.matmul_packed_weight_values(
+            unit, layer.packed_weight_indices, layer.row_norms, layer._weight_codebook_centroids,
+            bits=layer.weight_bits, out_features=layer.out_features, in_features=k, bias=layer.bias,
+            token_scale=flat_norms, output_dtype=x.dtype)
+    return fn
+
+
+def quantize_only_closure(layer, x):
+    from orbitquant_amd import ops
+
+    fmt = "nibble" if layer.activation_bits <= 4 else None
+    vals = None if fmt else "unit_bf16"
+
+    def fn():
+        return ops.rotate_quantize(
+            x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
+            block_size=layer.rotation.block_size, eps=layer.activation_eps,
+            inv_sqrt_block=layer.rotation.normalization, centroids=layer._activation_codebook_centroids,
+            code_format=fmt, values=vals)
+    return fn
+
+
+# ----------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(spec, layers, x, budget_rows):
+    """Oracle (CPU port of the reference path) on the first `budget_rows` tokens: per layer
+    rotate+quantize to values, then the scalar packed matmul with fp32 accumulation."""
+    from oracle import oracle_c, oracle_np
+
+    threads = oracle_c.max_threads()
+    rows = min(budget_rows, x.shape[0])
+    h = x[:rows].float().cpu().numpy()
+    flops = 0.0
+    prepared = []
+    for layer, act in layers:
+        prepared.append(dict(
+            perm=layer.rotation.permutation.numpy().astype(np.int32), signs=layer.rotation.signs.numpy(),
+            bounds=layer.activation_codebook.boundaries.numpy(), cents=layer.activation_codebook.centroids.numpy(),
+            block=layer.rotation.block_size, inv=np.float32(layer.rotation.normalization),
+            packed=layer.packed_weight_indices.cpu().numpy(), r=layer.row_norms.float().cpu().numpy(),
+            cw=layer.weight_codebook.centroids.numpy(), bits=layer.weight_bits, n=layer.out_features,
+            k=layer.in_features, act=act))
+    t0 = time.perf_counter()
+    for p in prepared:
+        codes, s = oracle_c.rotate_quantize(h, p["perm"], p["signs"], p["bounds"], p["block"], 1e-10, p["inv"], threads)
+        vals = p["cents"][codes] * s[:, None]
+        y = oracle_c.matmul_packed_weight(vals, p["packed"], p["r"], p["cw"], None, p["bits"], p["n"], threads)
+        flops += 2.0 * rows * p["n"] * p["k"]
+        if p["act"] == "gelu":
+            y = torch.nn.functional.gelu(torch.from_numpy(y)).numpy()
+        elif p["act"] == "slice3072":
+            y = np.ascontiguousarray(y[:, :3072])
+        h = y
+    dt = time.perf_counter() - t0
+    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=threads, kind="port",
+                sample=f"first {rows} of {x.shape[0]} tokens through every layer of the workload, {dt:.2f} s, "
+                       f"oracle/oq_oracle.c with OpenMP ({os.cpu_count()} logical CPUs visible)")
+
+
+# ------------------------------------------------------------------------ c5
+
+def build_c5(device, gen):
+    """The 240 distinct matrices of the 40-layer decode stack: per layer q,k (4096x4096), v,o
+    (4096x4096), up (14336x4096), down (4096x14336); interior layers q,k W2 and the rest W3,
+    first/last 4 layers all W4."""
+    from orbitquant_amd import OrbitLinear, OrbitQuantConfig
+
+    mats = []
+    for layer_idx in range(40):
+        boundary = layer_idx < 4 or layer_idx >= 36
+        for name, (k, n) in (("q", (4096, 4096)), ("k", (4096, 4096)), ("v", (4096, 4096)), ("o", (4096, 4096)),
+                             ("up", (4096, 14336)), ("down", (14336, 4096))):
+            bits = 4 if boundary else (2 if name in ("q", "k") else 3)
+            cfg = OrbitQuantConfig(weight_bits=bits, activation_bits=4)
+            packed = torch.randint(0, 256, ((n * k * bits + 7) // 8,), generator=gen, dtype=torch.uint8)
+            norms = torch.full((n,), 0.02 * np.sqrt(k)).to(torch.bfloat16)
+            mats.append(OrbitLinear(in_features=k, out_features=n, config=cfg, bias=None,
+                                    packed_weight_indices=packed, row_norms=norms).to(device))
+    return mats
+
+
+def bench_c5(args, device):
+    from orbitquant_amd import ops
+
+    gen = torch.Generator().manual_seed(5)
+    m = args.m or 1
+    mats = build_c5(device, gen)
+    x4096 = torch.randn(m, 4096, generator=gen).to(torch.bfloat16).to(device)
+    x14336 = torch.randn(m, 14336, generator=gen).to(torch.bfloat16).to(device)
+    packed_bytes = sum(l.packed_weight_indices.numel() + 2 * l.out_features for l in mats)
+    pre = []
+    for l in mats:
+        x = x4096 if l.in_features == 4096 else x14336
+        codes, _, norms = ops.rotate_quantize(
+            x, l._rotation_permutation, l._rotation_signs, l._activation_codebook_boundaries,
+            block_size=l.rotation.block_size, eps=l.activation_eps, inv_sqrt_block=l.rotation.normalization,
+            code_format="nibble")
+        pre.append((l, codes, norms))
+
+    def stack_matmuls():
+        for l, codes, norms in pre:
+            ops.packed_linear(codes, norms, l._activation_codebook_centroids, l.packed_weight_indices, l.row_norms,
+                              l._weight_codebook_centroids, code_format="nibble", activation_bits=4,
+                              weight_bits=l.weight_bits, out_features=l.out_features, in_features=l.in_features,
+                              output_dtype=torch.bfloat16)
+
+    def full_step():
+        for l in mats:
+            l(x4096 if l.in_features == 4096 else x14336)
+
+    for _ in range(args.warmup):
+        full_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        full_step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    # kernel-only: every matmul launch of the stack, events on the launch stream
+    per_stack = time_kernel(stack_matmuls, max(3, args.kernel_iters // 10))
+    # W4 matrices alone (the 8 boundary layers' MLP up projections), cycled so the cache cannot hold them
+    w4_up = [(l, c, n) for (l, c, n) in pre if l.weight_bits == 4 and l.out_features == 14336]
+
+    def w4_only():
+        for l, codes, norms in w4_up:
+            ops.packed_linear(codes, norms, l._activation_codebook_centroids, l.packed_weight_indices, l.row_norms,
+                              l._weight_codebook_centroids, code_format="nibble", activation_bits=4, weight_bits=4,
+                              out_features=l.out_features, in_features=l.in_features, output_dtype=torch.bfloat16)
+    per_w4 = time_kernel(w4_only, max(3, args.kernel_iters // 5)) / len(w4_up)
+    w4_bytes = w4_up[0][0].packed_weight_indices.numel() + 2 * 14336
+    achieved = w4_bytes / per_w4 / 1e9
+    out = {
+        "metric": "small-M packed-weight GB/s (whole decode stack, quantize + matmul per linear)",
+        "value": packed_bytes / dt / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": {"workload": f"c5 40-layer decode stack W2/W3/W4 A4, M={m}", "M": m,
+                                        "packed_bytes_per_step": packed_bytes},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "packed_gemv_kernel<4> on 4096->14336 W4", "bytes_per_launch": w4_bytes,
+                     "avg_launch_us": per_w4 * 1e6,
+                     "stack_matmuls_gbs": packed_bytes / per_stack / 1e9},
+    }
+    print(json.dumps(out))
+
+
+# ------------------------------------------------------------------------ main
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs an AMD GPU (the quantized-linear forward has no CPU fallback)", file=sys.stderr)
+        return 2
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    if args.workload == "c5":
+        bench_c5(args, device)
+        return 0
+
+    spec = workload_spec(args.workload, args.m)
+    gen = torch.Generator().manual_seed({"c1": 1, "c2": 2, "c3": 3, "c4": 4}[args.workload])
+    real = args.workload in ("c1", "c2")        # larger workloads: synthetic indices (weight quantization is offline)
+    layers = build_layers(spec, device, gen, real)
+    x = make_input(spec, spec["layers"][0][0], gen).to(device)
+    flops = sum(2.0 * spec["M"] * n * k for (k, n, *_rest) in spec["layers"])
+
+    for _ in range(args.warmup):
+        run_step(layers, x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step(layers, x)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    # dominant kernel alone: the packed GEMM of the first layer, and every other piece for the record
+    pieces = {}
+    h = x
+    for i, (layer, act) in enumerate(layers):
+        k, n = layer.in_features, layer.out_features
+        tq = time_kernel(quantize_only_closure(layer, h), args.kernel_iters)
+        tg = time_kernel(gemm_only_closure(layer, h), args.kernel_iters)
+        elem = 4 if h.dtype == torch.float32 else 2
+        q_bytes = spec["M"] * k * elem + spec["M"] * k * (0.5 if layer.activation_bits <= 4 else 2) + 4 * spec["M"]
+        pieces[f"layer{i}"] = {
+            "shape": [spec["M"], n, k], "gemm_us": tg * 1e6, "gemm_tflops": 2.0 * spec["M"] * n * k / tg / 1e12,
+            "quantize_us": tq * 1e6, "quantize_gbs": q_bytes / tq / 1e9}
+        h = run_step([(layer, act)], h)
+    dom = max(pieces.values(), key=lambda p: p["gemm_us"])
+    achieved = dom["gemm_tflops"]
+
+    out = {
+        "metric": "W4A4 packed-linear TFLOP/s (quantize + packed matmul, 2*M*N*K per linear)"
+        if args.workload in ("c1", "c2") else "packed-linear TFLOP/s (quantize + packed matmul, 2*M*N*K per linear)",
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": spec["name"], "M": spec["M"], "input_dtype": str(spec["dtype"]).replace("torch.", ""),
+                   "flop_per_step": flops},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "packed_gemm_kernel", "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},
+        "pieces": pieces,
+    }
+    if not args.no_cpu_baseline:
+        budget = {"c1": 256, "c2": 256, "c3": 48, "c4": 32}[args.workload]
+        out["cpu_baseline"] = cpu_baseline(spec, layers, x, budget)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

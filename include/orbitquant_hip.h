@@ -1,0 +1,145 @@
+/*
+ * orbitquant_hip.h - C ABI of the MI355X (gfx950) quantized-linear forward.
+ *
+ * One shared library, plain pointers and sizes, no framework types.  Every
+ * pointer is a DEVICE pointer unless a comment says otherwise; the library
+ * borrows them for the duration of the call and keeps nothing.  Work is
+ * enqueued on `stream` (a hipStream_t passed as void*; NULL = the null stream)
+ * and the call returns without synchronizing, so calls may be captured into a
+ * HIP graph.  Return value: OQ_OK or an oq_status error; `oq_last_error()`
+ * gives the text of the last error raised on the calling thread.
+ *
+ * The entry points replace, for AMD GPUs, the operators the reference's native
+ * package registers (paths relative to the reference checkout):
+ *   native-kernels/orbitquant-packed-matmul/torch-ext/torch_binding.cpp:7-66
+ *   native-kernels/orbitquant-packed-matmul/torch-ext/torch_binding.h:11-92
+ * and the kernels behind them in
+ *   native-kernels/orbitquant-packed-matmul/orbitquant_packed_matmul_cuda/packed_matmul.cu
+ */
+#ifndef ORBITQUANT_HIP_H
+#define ORBITQUANT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  OQ_OK = 0,
+  OQ_ERR_INVALID = 1,     /* an argument is out of its documented range        */
+  OQ_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for        */
+  OQ_ERR_LAUNCH = 3       /* the HIP runtime rejected a launch / attribute set */
+} oq_status;
+
+typedef enum { OQ_F32 = 0, OQ_F16 = 1, OQ_BF16 = 2 } oq_dtype;
+
+/* How activation codes are stored. */
+typedef enum {
+  OQ_CODES_U8 = 0,    /* one code per byte, [M, K]                                   */
+  OQ_CODES_NIBBLE = 1 /* two codes per byte, even k in the low nibble, [M, K/2];     */
+                      /* needs levels <= 16 and even K (packed_matmul.cu:648-656)    */
+} oq_code_format;
+
+/* What oq_rotate_quantize writes to `values_out`. */
+typedef enum {
+  OQ_VALUES_NONE = 0,
+  OQ_VALUES_SCALED = 1,  /* centroid[code] * ||x||, rounded to x's dtype, [M, K]     */
+                         /* (quantize_activations_cpu contract, torch_binding.h:28-37) */
+  OQ_VALUES_UNIT_BF16 = 2 /* bf16(centroid[code]), [M, K]; the token norm stays in   */
+                          /* norms_out and is applied by the matmul epilogue         */
+} oq_values_mode;
+
+/* Library / device probe.  Returns OQ_OK when a gfx950 device is current. */
+int oq_device_ok(void);
+const char *oq_last_error(void);
+const char *oq_version(void);
+
+/*
+ * Fused RPBH rotate + per-token quantize.
+ * Replaces quantize_activations_packed_w4 / quantize_activations_int8 /
+ * quantize_activations_cpu (torch_binding.cpp:13-31,47-66; kernels
+ * packed_matmul.cu:581-742; semantics src/orbitquant/functional.py:16-22):
+ *
+ *   s      = ||fp32(x_row)||_2                     (fixed summation order, see below)
+ *   unit   = fp32(x_row) / (s + eps)               (IEEE division)
+ *   y      = unit[perm] * signs                    (gather, exact)
+ *   y      = blockwise FWHT(y), block `block`, butterfly distance 1,2,4,...
+ *   rot    = y * inv_sqrt_block                    (one fp32 multiply)
+ *   code   = #{ j : boundaries[j] < rot }          (ties to the lower code)
+ *
+ * Sum of squares order: the row is zero-padded to a multiple of 2048 and viewed
+ * as [passes][256 lanes][8]; per (pass, lane) the eight squares are added as
+ * ((s0+s1)+(s2+s3))+((s4+s5)+(s6+s7)); each lane adds its passes left to right;
+ * the 256 lane sums are reduced by a balanced binary tree in lane order.  No
+ * operation is contracted into an FMA.
+ *
+ * x            [M, K] of x_dtype, row-major, contiguous
+ * perm         int32 [K], signs int8 [K] (+1/-1)
+ * boundaries   fp32 [levels-1], ascending;  2 <= levels <= 256
+ * centroids    fp32 [levels]; only read when values_mode != OQ_VALUES_NONE (else may be NULL)
+ * block        power of two dividing K;  K <= 16384
+ * codes_out    NULL or [M, K] u8 / [M, K/2] u8 per code_format
+ * values_out   NULL or per values_mode
+ * norms_out    fp32 [M]: the raw norm s (no eps); may be NULL
+ */
+int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K,
+                       const int32_t *perm, const int8_t *signs,
+                       const float *boundaries, const float *centroids, int levels,
+                       int64_t block, float eps, float inv_sqrt_block,
+                       void *codes_out, int code_format,
+                       void *values_out, int values_mode,
+                       float *norms_out, void *stream);
+
+/*
+ * Packed-weight linear on quantized activations (the fused hot path):
+ *
+ *   out[m,n] = (sum_k c_a[code[m,k]] * c_w[idx[n,k]]) * s[m] * r_w[n] + bias[n]
+ *
+ * Replaces matmul_packed_w4a4_int8 (torch_binding.cpp:39-46; packed_matmul.cu:744-1009)
+ * for every weight width, with exact (bf16-rounded) centroids instead of the
+ * int8 surrogate.  M <= 16 takes the streaming small-M kernel, larger M the MFMA
+ * tile kernel.
+ *
+ * codes        activation codes in code_format (see oq_rotate_quantize)
+ * token_norms  fp32 [M]
+ * act_centroids fp32 [2^a_bits]
+ * packed_w     flat little-endian bit stream of idx[N,K], value v at bits [v*w_bits, v*w_bits+w_bits)
+ *              (src/orbitquant/packing/bitpack.py:8-46); w_bits in {2,3,4,6,8}
+ * row_norms    bf16 [N] (raw uint16 bit patterns)
+ * w_centroids  fp32 [2^w_bits]
+ * bias         NULL or [N] of bias_dtype
+ * out          [M, N] of out_dtype (OQ_BF16, OQ_F16 or OQ_F32)
+ */
+int oq_packed_linear(const void *codes, int code_format, const float *token_norms,
+                     const float *act_centroids, int a_bits,
+                     const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                     const float *w_centroids, const void *bias, int bias_dtype,
+                     int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                     void *stream);
+
+/*
+ * Packed-weight matmul on float activations:
+ *
+ *   out[m,n] = (sum_k x[m,k] * c_w[idx[n,k]]) * r_w[n] + bias[n]      (out in x's dtype)
+ *
+ * Replaces matmul_packed_weight (torch_binding.cpp:7-12,32-38; packed_matmul.cu:1335-1713).
+ * bits in [1, 8].  token_scale: NULL, or fp32 [M] multiplied into row m (lets the
+ * caller pass unit-norm bf16 centroids plus token norms).
+ */
+int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale,
+                            const uint8_t *packed_w, int bits, const uint16_t *row_norms,
+                            const float *w_centroids, const void *bias, int bias_dtype,
+                            int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                            void *stream);
+
+/*
+ * Unpack a little-endian bit stream into one index per byte (debug / tests;
+ * the GPU twin of unpack_lowbit, src/orbitquant/packing/bitpack.py:63-97).
+ */
+int oq_unpack_lowbit(const uint8_t *packed, int bits, int64_t count, uint8_t *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ORBITQUANT_HIP_H */

@@ -1,0 +1,148 @@
+// extern "C" entry points: argument validation and kernel selection.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "oq_common.h"
+
+namespace oq {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int fail(oq_status code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return static_cast<int>(code);
+}
+
+int check_launch(const char *what) {
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return fail(OQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
+  return OQ_OK;
+}
+
+// kernels (defined in the other translation units)
+int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
+                             const int8_t *signs, const float *boundaries, const float *centroids,
+                             int levels, int64_t block, float eps, float inv_sqrt_block,
+                             void *codes_out, int code_format, void *values_out, int values_mode,
+                             float *norms_out, hipStream_t stream);
+int generic_matmul_float(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
+                         int bits, const uint16_t *row_norms, const float *w_cents, const void *bias,
+                         int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                         hipStream_t stream);
+int generic_linear_codes(const void *codes, int code_format, const float *token_norms,
+                         const float *act_cents, int a_levels, const uint8_t *packed_w, int bits,
+                         const uint16_t *row_norms, const float *w_cents, const void *bias,
+                         int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                         hipStream_t stream);
+int unpack_dispatch(const uint8_t *packed, int bits, int64_t count, uint8_t *out, hipStream_t stream);
+bool gemm_supported(int64_t K, int bits);
+int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
+                  const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
+                  const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
+                  int out_dtype, hipStream_t stream);
+bool gemv_supported(int64_t M, int64_t K, int bits, int code_format, int a_levels);
+int gemv_dispatch(const void *codes, const float *row_scale, const float *act_cents, int a_levels,
+                  const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
+                  const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
+                  int out_dtype, hipStream_t stream);
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static bool valid_dtype(int dt) { return dt == OQ_F32 || dt == OQ_F16 || dt == OQ_BF16; }
+
+static int check_matmul_common(const char *who, const uint8_t *packed_w, int bits, const uint16_t *row_norms,
+                               const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N,
+                               int64_t K, const void *out, int out_dtype) {
+  if (M < 0 || N <= 0 || K <= 0) return fail(OQ_ERR_INVALID, "%s: M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
+  if (bits < 1 || bits > 8) return fail(OQ_ERR_INVALID, "%s: bits=%d not in [1, 8]", who, bits);
+  if (packed_w == nullptr || row_norms == nullptr || w_cents == nullptr || (out == nullptr && M > 0))
+    return fail(OQ_ERR_INVALID, "%s: null pointer", who);
+  if (!valid_dtype(out_dtype)) return fail(OQ_ERR_INVALID, "%s: out_dtype=%d", who, out_dtype);
+  if (bias != nullptr && !valid_dtype(bias_dtype)) return fail(OQ_ERR_INVALID, "%s: bias_dtype=%d", who, bias_dtype);
+  return OQ_OK;
+}
+
+}  // namespace oq
+
+using namespace oq;
+
+extern "C" {
+
+const char *oq_last_error(void) { return g_error; }
+
+const char *oq_version(void) { return "orbitquant-hip 0.1 (gfx950)"; }
+
+int oq_device_ok(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(OQ_ERR_LAUNCH, "no HIP device is current");
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return fail(OQ_ERR_LAUNCH, "cannot query device %d", dev);
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(OQ_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+  return OQ_OK;
+}
+
+int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
+                       const int8_t *signs, const float *boundaries, const float *centroids, int levels,
+                       int64_t block, float eps, float inv_sqrt_block, void *codes_out, int code_format,
+                       void *values_out, int values_mode, float *norms_out, void *stream) {
+  return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
+                                  inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
+                                  as_stream(stream));
+}
+
+int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
+                     int a_bits, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                     const float *w_centroids, const void *bias, int bias_dtype, int64_t M, int64_t N,
+                     int64_t K, void *out, int out_dtype, void *stream) {
+  if (int rc = check_matmul_common("packed_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
+  if (M == 0) return OQ_OK;
+  if (codes == nullptr || act_centroids == nullptr) return fail(OQ_ERR_INVALID, "packed_linear: null codes/centroids");
+  if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "packed_linear: a_bits=%d", a_bits);
+  if (code_format != OQ_CODES_U8 && code_format != OQ_CODES_NIBBLE) return fail(OQ_ERR_INVALID, "packed_linear: code_format=%d", code_format);
+  if (code_format == OQ_CODES_NIBBLE && (a_bits > 4 || (K & 1))) return fail(OQ_ERR_INVALID, "packed_linear: nibble codes need a_bits <= 4 and even K");
+  const int a_levels = 1 << a_bits;
+  hipStream_t s = as_stream(stream);
+  const bool fast_ptrs = aligned16(codes) && aligned16(packed_w);
+  if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
+    return gemv_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
+                         bias, bias_dtype, M, N, K, out, out_dtype, s);
+  if (fast_ptrs && code_format == OQ_CODES_NIBBLE && gemm_supported(K, w_bits))
+    return gemm_dispatch(0, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
+                         bias, bias_dtype, M, N, K, out, out_dtype, s);
+  return generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
+                              w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+}
+
+int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
+                            int bits, const uint16_t *row_norms, const float *w_centroids, const void *bias,
+                            int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                            void *stream) {
+  if (int rc = check_matmul_common("matmul_packed_weight", packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
+  if (M == 0) return OQ_OK;
+  if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
+  hipStream_t s = as_stream(stream);
+  if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_supported(K, bits))
+    return gemm_dispatch(x_dtype == OQ_BF16 ? 1 : 2, x, token_scale, nullptr, 0, packed_w, bits, row_norms,
+                         w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+  return generic_matmul_float(x, x_dtype, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N,
+                              K, out, out_dtype, s);
+}
+
+int oq_unpack_lowbit(const uint8_t *packed, int bits, int64_t count, uint8_t *out, void *stream) {
+  if (bits < 1 || bits > 8 || count < 0) return fail(OQ_ERR_INVALID, "unpack_lowbit: bits=%d count=%lld", bits, (long long)count);
+  if (count > 0 && (packed == nullptr || out == nullptr)) return fail(OQ_ERR_INVALID, "unpack_lowbit: null pointer");
+  return unpack_dispatch(packed, bits, count, out, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,260 @@
+// Packed-weight GEMM on the gfx950 matrix cores.
+//
+//   out[m,n] = (sum_k A[m,k] * c_w[idx[n,k]]) * scale[m] * r_w[n] + bias[n]
+//
+// A is either packed 4-bit activation codes (decoded through a codebook table)
+// or 16-bit float values; idx is the flat little-endian bit stream of 2/3/4/6/8
+// bit weight indices, read from HBM as it is stored.  Nothing is dequantized to
+// memory: every wavefront loads the packed dwords of its own rows straight into
+// registers, turns them into bf16 MFMA operands through lookup tables held in
+// LDS, and feeds v_mfma_f32_32x32x16_bf16.
+//
+// Operand layout.  One MFMA consumes, per lane, eight k-values of one row
+// (lane l: row l%32, k-group l/32).  A dot product does not care in which order
+// k is visited as long as both operands agree, so a K-step of 64 is cut as
+//   lane group g (0/1) owns k0+32g .. k0+32g+31   (one contiguous run of bits per row)
+//   MFMA q (0..3) of the step uses values 8q..8q+7 of that run
+// which makes every global load of packed data one contiguous 4*bits-byte run
+// per lane (16 bytes for 4-bit), with no cross-lane shuffles and no LDS staging.
+//
+// Lookup tables.  Two codes are decoded per LDS read: the table is indexed by
+// the 2*bits-bit pair and returns both bf16 values in one dword.  Tables of up
+// to 256 pairs are replicated 32 times so that lane l reads copy l%32 and a
+// wavefront never has two different addresses in one LDS bank.
+#include "packed_decode.h"
+
+namespace oq {
+namespace {
+
+enum AMode { A_NIBBLE = 0, A_BF16 = 1, A_F16 = 2 };
+
+struct GemmArgs {
+  const uint8_t *a;          // [M, K/2] nibble codes or [M, K] 16-bit floats
+  const float *row_scale;    // [M] or NULL
+  const float *act_cents;    // [16] (nibble mode)
+  int a_levels;
+  const uint8_t *w;          // packed index stream
+  const uint16_t *row_norms; // bf16 [N]
+  const float *w_cents;      // [2^bits]
+  const void *bias;
+  int bias_dtype;
+  int64_t M, N, K;
+  void *out;
+  int out_dtype;
+  int tiles_m, tiles_n;
+};
+
+template <int AM> struct ARaw { uint4 v[AM == A_NIBBLE ? 1 : 4]; };
+
+template <int AM>
+__device__ __forceinline__ void load_a(const uint8_t *p, ARaw<AM> &r) {
+  const uint4 *q = reinterpret_cast<const uint4 *>(p);
+#pragma unroll
+  for (int i = 0; i < (AM == A_NIBBLE ? 1 : 4); ++i) r.v[i] = q[i];
+}
+
+template <int AM>
+__device__ __forceinline__ f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+  if constexpr (AM == A_F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Workgroup = 4 wavefronts in a 2x2 arrangement; each wavefront owns FM x FN MFMA tiles of 32x32.
+template <int AM, int BITS, int FM, int FN>
+__global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
+  extern __shared__ __align__(16) uint32_t lds[];
+  uint32_t *wlut = lds;
+  uint32_t *alut = lds + WLut<BITS>::kDwords;
+
+  fill_pair_lut<AM == A_F16>(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPairBits, WLut<BITS>::kLogRep, BITS == 8);
+  if constexpr (AM == A_NIBBLE) fill_pair_lut<false>(alut, g.act_cents, 4, g.a_levels, 8, kALutLogRep, false);
+  __syncthreads();
+
+  constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
+  // tile order: spread consecutive workgroup ids over the 8 XCDs' private L2s in
+  // contiguous chunks, then walk groups of 4 tile-rows column by column
+  int bid = blockIdx.x;
+  const int total = g.tiles_m * g.tiles_n;
+  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
+  constexpr int GROUP_M = 4;
+  const int width = GROUP_M * g.tiles_n;
+  const int group = bid / width;
+  const int first_m = group * GROUP_M;
+  const int gsz = min(g.tiles_m - first_m, GROUP_M);
+  const int pid_m = first_m + (bid % width) % gsz;
+  const int pid_n = (bid % width) / gsz;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, grp = lane >> 5, rl = lane & 31;
+  const int64_t m_base = static_cast<int64_t>(pid_m) * TM + (wave >> 1) * (FM * 32);
+  const int64_t n_base = static_cast<int64_t>(pid_n) * TN + (wave & 1) * (FN * 32);
+
+  constexpr int A_ROW_STEP = AM == A_NIBBLE ? 32 : 128;  // bytes of one row consumed per K-step of 64
+  constexpr int A_GRP_OFF = AM == A_NIBBLE ? 16 : 64;
+  const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K * 2;
+  const int64_t w_row_bytes = g.K * BITS / 8;
+
+  const uint8_t *ap[FM];
+  const uint8_t *wp[FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int64_t row = min(m_base + 32 * i + r, g.M - 1);
+    ap[i] = g.a + row * a_row_bytes + grp * A_GRP_OFF;
+  }
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+    const int64_t row = min(n_base + 32 * j + r, g.N - 1);
+    wp[j] = g.w + row * w_row_bytes + grp * (4 * BITS);
+  }
+
+  f32x16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  ARaw<AM> a_nxt[FM];
+  uint32_t w_nxt[FN][BITS];
+#pragma unroll
+  for (int i = 0; i < FM; ++i) load_a<AM>(ap[i], a_nxt[i]);
+#pragma unroll
+  for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j], w_nxt[j]);
+
+  const int steps = static_cast<int>(g.K / 64);
+  for (int ks = 0; ks < steps; ++ks) {
+    ARaw<AM> a_cur[FM];
+    uint32_t w_cur[FN][BITS];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) a_cur[i] = a_nxt[i];
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int d = 0; d < BITS; ++d) w_cur[j][d] = w_nxt[j][d];
+    if (ks + 1 < steps) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + static_cast<int64_t>(ks + 1) * A_ROW_STEP, a_nxt[i]);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(ks + 1) * (8 * BITS), w_nxt[j]);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint4 af[FM], bf[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        if constexpr (AM == A_NIBBLE) {
+          const uint32_t f = q == 0 ? a_cur[i].v[0].x : q == 1 ? a_cur[i].v[0].y : q == 2 ? a_cur[i].v[0].z : a_cur[i].v[0].w;
+          af[i] = decode_a_nibble(f, alut, rl);
+        } else {
+          af[i] = a_cur[i].v[q];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bf[j] = decode_w<BITS>(w_cur[j], q, wlut, rl);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(af[i], bf[j], acc[i][j]);
+    }
+  }
+
+  // ---- epilogue: acc * scale[m] * r_w[n] + bias[n] ------------------------------
+  // accumulator e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 of its 32x32 tile
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+    const int64_t n = n_base + 32 * j + r;
+    if (n >= g.N) continue;
+    const float rn = bf16_bits_to_f32(g.row_norms[n]);
+    const float bv = g.bias != nullptr ? load_dyn_f32(g.bias, g.bias_dtype, n) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t m = m_base + 32 * i + 8 * (e >> 2) + 4 * grp + (e & 3);
+        if (m >= g.M) continue;
+        const float sc = g.row_scale != nullptr ? g.row_scale[m] : 1.0f;
+        const float y = acc[i][j][e] * sc * rn + bv;
+        const int64_t o = m * g.N + n;
+        if (g.out_dtype == OQ_BF16) static_cast<uint16_t *>(g.out)[o] = f32_to_bf16_bits(y);
+        else if (g.out_dtype == OQ_F16) static_cast<uint16_t *>(g.out)[o] = f32_to_f16_bits(y);
+        else static_cast<float *>(g.out)[o] = y;
+      }
+    }
+  }
+}
+
+template <int AM, int BITS, int FM, int FN>
+int launch_cfg(GemmArgs g, hipStream_t stream) {
+  constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
+  g.tiles_m = static_cast<int>((g.M + TM - 1) / TM);
+  g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
+  const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
+  if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
+  const size_t smem = (WLut<BITS>::kDwords + (AM == A_NIBBLE ? kALutDwords : 0)) * sizeof(uint32_t);
+  auto kern = packed_gemm_kernel<AM, BITS, FM, FN>;
+  if (smem > 48 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(smem)) != hipSuccess)
+      return fail(OQ_ERR_LAUNCH, "packed_gemm: cannot reserve %zu bytes of LDS", smem);
+  }
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), smem, stream, g);
+  return check_launch("packed_gemm");
+}
+
+template <int AM, int BITS>
+int launch_bits(const GemmArgs &g, int tile, hipStream_t stream) {
+  if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
+  if (tile == 1) return launch_cfg<AM, BITS, 2, 4>(g, stream);
+  return launch_cfg<AM, BITS, 2, 2>(g, stream);
+}
+
+template <int AM>
+int launch_mode(const GemmArgs &g, int bits, int tile, hipStream_t stream) {
+  switch (bits) {
+    case 2: return launch_bits<AM, 2>(g, tile, stream);
+    case 3: return launch_bits<AM, 3>(g, tile, stream);
+    case 4: return launch_bits<AM, 4>(g, tile, stream);
+    case 6: return launch_bits<AM, 6>(g, tile, stream);
+    case 8: return launch_bits<AM, 8>(g, tile, stream);
+    default: return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: weight width %d", bits);
+  }
+}
+
+// Tile choice: the largest tile that still gives every CU work.
+int choose_tile(int64_t M, int64_t N) {
+  const char *force = getenv("OQ_GEMM_TILE");
+  if (force != nullptr && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
+  auto tiles = [&](int tm, int tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
+  if (tiles(256, 256) >= 512) return 2;
+  if (tiles(128, 256) >= 384) return 1;
+  return 0;
+}
+
+}  // namespace
+
+bool gemm_supported(int64_t K, int bits) {
+  return K % 64 == 0 && (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
+}
+
+// a_mode: 0 nibble codes, 1 bf16 values, 2 fp16 values
+int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
+                  const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
+                  const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
+                  int out_dtype, hipStream_t stream) {
+  GemmArgs g{};
+  g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
+  g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
+  g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
+  const int tile = choose_tile(M, N);
+  switch (a_mode) {
+    case A_NIBBLE: return launch_mode<A_NIBBLE>(g, bits, tile, stream);
+    case A_BF16: return launch_mode<A_BF16>(g, bits, tile, stream);
+    case A_F16: return launch_mode<A_F16>(g, bits, tile, stream);
+    default: return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
+  }
+}
+
+}  // namespace oq

@@ -1,0 +1,175 @@
+"""`OrbitLinear`: the quantized linear module, MI355X path.
+
+State dict = `packed_weight_indices` (uint8, flat bit stream), `row_norms`
+(bfloat16 [N]) and `bias`, exactly the reference module's persistent tensors
+(src/orbitquant/layers.py:386-400); rotation / codebook constants are
+non-persistent buffers rebuilt from (in_features, seed, block, bits)
+(layers.py:358-385,625-649).
+
+Forward = one opaque custom op (`orbitquant_amd::quantized_linear`) with a fake
+implementation, so `torch.compile(fullgraph=True)` traces through it the way
+the reference's `orbitquant::packed_linear_forward` does (layers.py:38-72,
+1072-1077).  The op is stateless: every tensor it needs is an argument.
+
+Inside the op (the reference's `_forward_impl`, layers.py:1079-1455, for AMD):
+  1. fused rotate + per-token quantize (HIP) -> activation codes + token norms
+  2. packed-weight matmul (HIP): streaming kernel for <= 16 tokens, MFMA tile
+     kernel otherwise; activation widths above 4 bits hand the matmul bf16
+     centroid values instead of nibble codes.
+There is no dequantized-weight or CPU fallback on this path.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from . import ops
+from .codebooks import get_codebook
+from .config import OrbitQuantConfig
+from .rotations import get_rpbh_rotation
+from .weights import quantize_weight
+
+_LIB = torch.library.Library("orbitquant_amd", "DEF")
+_LIB.define(
+    "quantized_linear(Tensor x, Tensor permutation, Tensor signs, Tensor act_centroids, "
+    "Tensor act_boundaries, Tensor packed_weight_indices, Tensor row_norms, Tensor weight_centroids, "
+    "Tensor? bias, int block_size, float eps, float inv_sqrt_block, int activation_bits, "
+    "int weight_bits, int out_features) -> Tensor"
+)
+
+
+def quantized_linear_forward(
+    x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
+    weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
+):
+    in_features = x.shape[-1]
+    if bias is not None and bias.dtype != x.dtype:
+        bias = bias.to(x.dtype)
+    if activation_bits <= 4 and in_features % 2 == 0:
+        codes, _, norms = ops.rotate_quantize(
+            x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
+            inv_sqrt_block=inv_sqrt_block, code_format="nibble")
+        return ops.packed_linear(
+            codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
+            code_format="nibble", activation_bits=activation_bits, weight_bits=weight_bits,
+            out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
+    _, unit, norms = ops.rotate_quantize(
+        x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
+        inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16")
+    return ops.matmul_packed_weight_values(
+        unit, packed_weight_indices, row_norms, weight_centroids, bits=weight_bits,
+        out_features=out_features, in_features=in_features, bias=bias,
+        token_scale=norms.reshape(-1), output_dtype=x.dtype)
+
+
+def _quantized_linear_fake(
+    x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
+    weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
+):
+    return x.new_empty((*x.shape[:-1], out_features))
+
+
+_LIB.impl("quantized_linear", quantized_linear_forward, "CUDA")
+torch.library.register_fake("orbitquant_amd::quantized_linear", _quantized_linear_fake, lib=_LIB)
+
+
+def packed_length(value_count: int, bits: int) -> int:
+    return (value_count * bits + 7) // 8
+
+
+class OrbitLinear(nn.Module):
+    def __init__(
+        self,
+        *,
+        in_features: int,
+        out_features: int,
+        config: OrbitQuantConfig,
+        bias: torch.Tensor | None,
+        packed_weight_indices: torch.Tensor,
+        row_norms: torch.Tensor,
+        module_name: str = "",
+    ) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight_bits = config.weight_bits
+        self.activation_bits = config.activation_bits
+        self.activation_eps = config.activation_eps
+        self.module_name = module_name
+        self.rotation = get_rpbh_rotation(in_features, config.rotation_seed, config.block_size)
+        self.weight_codebook = get_codebook(in_features, config.weight_bits, config.codebook_version)
+        self.activation_codebook = get_codebook(in_features, config.activation_bits, config.codebook_version)
+        expected = packed_length(out_features * in_features, config.weight_bits)
+        if packed_weight_indices.dtype != torch.uint8 or packed_weight_indices.numel() != expected:
+            raise ValueError(f"packed_weight_indices must be uint8 with {expected} bytes")
+        if row_norms.dtype != torch.bfloat16 or tuple(row_norms.shape) != (out_features,):
+            raise ValueError("row_norms must be bfloat16 with shape (out_features,)")
+        self.packed_weight_indices = nn.Parameter(packed_weight_indices.detach().flatten(), requires_grad=False)
+        self.row_norms = nn.Parameter(row_norms.detach(), requires_grad=False)
+        if bias is None:
+            self.register_parameter("bias", None)
+        else:
+            self.bias = nn.Parameter(bias.detach().clone(), requires_grad=False)
+        device = packed_weight_indices.device
+        for name, tensor in self._constants().items():
+            self.register_buffer(name, tensor.to(device), persistent=False)
+        self.last_effective_runtime_mode: str | None = None
+
+    def _constants(self) -> dict[str, torch.Tensor]:
+        return {
+            "_rotation_permutation": self.rotation.permutation.to(torch.int32),
+            "_rotation_signs": self.rotation.signs.to(torch.int8),
+            "_activation_codebook_centroids": self.activation_codebook.centroids.clone(),
+            "_activation_codebook_boundaries": self.activation_codebook.boundaries.clone(),
+            "_weight_codebook_centroids": self.weight_codebook.centroids.clone(),
+        }
+
+    @classmethod
+    def from_weight(cls, weight, *, bias, config: OrbitQuantConfig, module_name: str = "") -> "OrbitLinear":
+        out_features, in_features = weight.shape
+        rotation = get_rpbh_rotation(in_features, config.rotation_seed, config.block_size)
+        codebook = get_codebook(in_features, config.weight_bits, config.codebook_version)
+        packed, row_norms = quantize_weight(
+            weight, rotation=rotation, codebook=codebook, bits=config.weight_bits,
+            eps=config.activation_eps, row_tile=config.weight_row_tile_size)
+        device = weight.device
+        return cls(
+            in_features=in_features, out_features=out_features, config=config,
+            bias=None if bias is None else bias.detach(),
+            packed_weight_indices=packed.to(device), row_norms=row_norms.to(device),
+            module_name=module_name)
+
+    @classmethod
+    def from_linear(cls, layer: nn.Linear, *, config: OrbitQuantConfig, module_name: str = "") -> "OrbitLinear":
+        if not isinstance(layer, nn.Linear):
+            raise TypeError(f"no OrbitQuant linear adapter registered for {type(layer).__name__}")
+        return cls.from_weight(layer.weight.detach(), bias=layer.bias, config=config, module_name=module_name)
+
+    def _apply(self, fn, recurse: bool = True):
+        result = super()._apply(fn, recurse=recurse)
+        # integer / fp32 constants must survive .to(dtype=...) casts unchanged
+        device = self.packed_weight_indices.device
+        for name, tensor in self._constants().items():
+            setattr(self, name, tensor.to(device))
+        return result
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.shape[-1] != self.in_features:
+            raise ValueError(f"expected last dimension {self.in_features}, got {x.shape[-1]}")
+        if x.device.type != "cuda":
+            raise RuntimeError(
+                "OrbitLinear runs on AMD GPUs only (torch device 'cuda'); there is no CPU fallback")
+        if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            raise ValueError("x must be float32, float16 or bfloat16")
+        self.last_effective_runtime_mode = "hip_packed"
+        return torch.ops.orbitquant_amd.quantized_linear(
+            x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_centroids,
+            self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
+            self._weight_codebook_centroids, self.bias, self.rotation.block_size,
+            self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
+            self.out_features)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"w{self.weight_bits}a{self.activation_bits}, block={self.rotation.block_size}")

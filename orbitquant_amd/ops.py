@@ -1,0 +1,188 @@
+"""torch-tensor front end of the C ABI: allocation, dtype plumbing, stream.
+
+The wrappers own allocation (as the reference's Python wrappers do,
+native-kernels/orbitquant-packed-matmul/torch-ext/orbitquant_packed_matmul/__init__.py:130-160),
+pass raw device pointers and the current HIP stream, and never synchronize.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import (OQ_BF16, OQ_CODES_NIBBLE, OQ_CODES_U8, OQ_F16, OQ_F32, OQ_VALUES_NONE,
+                   OQ_VALUES_SCALED, OQ_VALUES_UNIT_BF16)
+
+_DTYPES = {torch.float32: OQ_F32, torch.float16: OQ_F16, torch.bfloat16: OQ_BF16}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {t.dtype}") from None
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError(f"{name} must live on an AMD GPU (torch device 'cuda'); got {t.device}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def rotate_quantize(
+    x: torch.Tensor,
+    permutation: torch.Tensor,
+    signs: torch.Tensor,
+    boundaries: torch.Tensor,
+    *,
+    block_size: int,
+    eps: float,
+    inv_sqrt_block: float,
+    centroids: torch.Tensor | None = None,
+    code_format: str | None = "u8",
+    values: str | None = None,
+) -> tuple[torch.Tensor | None, torch.Tensor | None, torch.Tensor]:
+    """-> (codes or None, values or None, norms[...]).
+
+    code_format: "u8" ([..., K] uint8), "nibble" ([..., K/2] uint8) or None.
+    values: None, "scaled" (centroid*norm in x.dtype) or "unit_bf16" (bf16 centroid).
+    permutation int32, signs int8, boundaries/centroids fp32, all on x's device.
+    """
+    _require_gpu(x, "x")
+    dim = x.shape[-1]
+    rows = x.contiguous().reshape(-1, dim)
+    m = rows.shape[0]
+    lead = x.shape[:-1]
+    levels = boundaries.numel() + 1
+    if permutation.dtype != torch.int32 or signs.dtype != torch.int8:
+        raise ValueError("permutation must be int32 and signs int8")
+    if boundaries.dtype != torch.float32 or (centroids is not None and centroids.dtype != torch.float32):
+        raise ValueError("boundaries and centroids must be float32")
+    codes = None
+    fmt = OQ_CODES_U8
+    if code_format == "u8":
+        codes = torch.empty((m, dim), dtype=torch.uint8, device=x.device)
+    elif code_format == "nibble":
+        fmt = OQ_CODES_NIBBLE
+        codes = torch.empty((m, dim // 2), dtype=torch.uint8, device=x.device)
+    elif code_format is not None:
+        raise ValueError(f"unknown code_format {code_format!r}")
+    out_values = None
+    mode = OQ_VALUES_NONE
+    if values == "scaled":
+        mode = OQ_VALUES_SCALED
+        out_values = torch.empty_like(rows)
+    elif values == "unit_bf16":
+        mode = OQ_VALUES_UNIT_BF16
+        out_values = torch.empty((m, dim), dtype=torch.bfloat16, device=x.device)
+    elif values is not None:
+        raise ValueError(f"unknown values mode {values!r}")
+    if mode != OQ_VALUES_NONE and centroids is None:
+        raise ValueError("centroids are required when values are requested")
+    norms = torch.empty(m, dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.oq_rotate_quantize(
+            rows.data_ptr(), _dt(rows), m, dim, permutation.data_ptr(), signs.data_ptr(),
+            boundaries.data_ptr(), _ptr(centroids), levels, int(block_size), float(eps),
+            float(inv_sqrt_block), _ptr(codes), fmt, _ptr(out_values), mode, norms.data_ptr(),
+            _stream(x))
+    _lib.check(rc, "oq_rotate_quantize")
+    if codes is not None:
+        codes = codes.reshape(*lead, codes.shape[-1])
+    if out_values is not None:
+        out_values = out_values.reshape(*lead, dim)
+    return codes, out_values, norms.reshape(lead)
+
+
+def packed_linear(
+    codes: torch.Tensor,
+    token_norms: torch.Tensor,
+    activation_centroids: torch.Tensor,
+    packed_weight_indices: torch.Tensor,
+    row_norms: torch.Tensor,
+    weight_centroids: torch.Tensor,
+    *,
+    code_format: str,
+    activation_bits: int,
+    weight_bits: int,
+    out_features: int,
+    in_features: int,
+    bias: torch.Tensor | None = None,
+    output_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    _require_gpu(codes, "codes")
+    fmt = {"u8": OQ_CODES_U8, "nibble": OQ_CODES_NIBBLE}[code_format]
+    width = in_features if fmt == OQ_CODES_U8 else in_features // 2
+    if codes.dtype != torch.uint8 or codes.shape[-1] != width:
+        raise ValueError(f"codes must be uint8 with last dimension {width}")
+    lead = codes.shape[:-1]
+    flat = codes.contiguous().reshape(-1, width)
+    m = flat.shape[0]
+    if row_norms.dtype != torch.bfloat16 or packed_weight_indices.dtype != torch.uint8:
+        raise ValueError("row_norms must be bfloat16 and packed_weight_indices uint8")
+    expected = (out_features * in_features * weight_bits + 7) // 8
+    if packed_weight_indices.numel() < expected:
+        raise ValueError(f"packed_weight_indices holds {packed_weight_indices.numel()} bytes, needs {expected}")
+    out = torch.empty((m, out_features), dtype=output_dtype, device=codes.device)
+    norms = token_norms.reshape(-1)
+    if norms.dtype != torch.float32 or norms.numel() != m:
+        raise ValueError("token_norms must be float32 with one entry per token")
+    lib = _lib.load()
+    with torch.cuda.device(codes.device):
+        rc = lib.oq_packed_linear(
+            flat.data_ptr(), fmt, norms.contiguous().data_ptr(), activation_centroids.data_ptr(),
+            int(activation_bits), packed_weight_indices.data_ptr(), int(weight_bits),
+            row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
+            _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
+            out.data_ptr(), _DTYPES[output_dtype], _stream(codes))
+    _lib.check(rc, "oq_packed_linear")
+    return out.reshape(*lead, out_features)
+
+
+def matmul_packed_weight_values(
+    x: torch.Tensor,
+    packed_weight_indices: torch.Tensor,
+    row_norms: torch.Tensor,
+    weight_centroids: torch.Tensor,
+    *,
+    bits: int,
+    out_features: int,
+    in_features: int,
+    bias: torch.Tensor | None = None,
+    token_scale: torch.Tensor | None = None,
+    output_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    _require_gpu(x, "x")
+    lead = x.shape[:-1]
+    flat = x.contiguous().reshape(-1, in_features)
+    m = flat.shape[0]
+    out_dtype = x.dtype if output_dtype is None else output_dtype
+    out = torch.empty((m, out_features), dtype=out_dtype, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.oq_matmul_packed_weight(
+            flat.data_ptr(), _dt(flat), _ptr(token_scale), packed_weight_indices.data_ptr(), int(bits),
+            row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
+            _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
+            out.data_ptr(), _DTYPES[out_dtype], _stream(x))
+    _lib.check(rc, "oq_matmul_packed_weight")
+    return out.reshape(*lead, out_features)
+
+
+def unpack_lowbit(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
+    _require_gpu(packed, "packed")
+    out = torch.empty(length, dtype=torch.uint8, device=packed.device)
+    lib = _lib.load()
+    with torch.cuda.device(packed.device):
+        rc = lib.oq_unpack_lowbit(packed.contiguous().data_ptr(), int(bits), int(length), out.data_ptr(),
+                                  _stream(packed))
+    _lib.check(rc, "oq_unpack_lowbit")
+    return out

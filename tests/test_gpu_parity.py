@@ -1,0 +1,400 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle.
+
+Bars: activation codes, token norms and packed-index decode bit-exact; matmul
+outputs within max-abs-error <= 2e-2 * ||x|| * ||w_row|| / sqrt(K) per element and
+cosine similarity >= 0.9999 against the fp64 statement of the dequantized path.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle_c, oracle_np as o
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("needs an AMD GPU")
+    from orbitquant_amd import _lib
+
+    lib = _lib.load()
+    assert lib.oq_device_ok() == 0, lib.oq_last_error()
+    return torch.device("cuda:0")
+
+
+_TABLES: dict = {}
+
+
+def tables(dim, bits):
+    key = (dim, bits)
+    if key not in _TABLES:
+        _TABLES[key] = o.lloyd_max_tables(dim, bits)
+    return _TABLES[key]
+
+
+def make_x(rng, m, k, dtype, kind="outliers"):
+    x = rng.standard_normal((m, k)).astype(F32)
+    if kind == "outliers":
+        x[rng.random(x.shape) < 0.01] *= 20
+    elif kind == "student":
+        x = rng.standard_t(4, size=(m, k)).astype(F32)
+    t = torch.from_numpy(x).to(dtype)
+    return t, t.float().numpy()
+
+
+def gpu_rotate_quantize(dev, xt, perm, signs, bounds, block, eps, inv, cents=None, fmt="u8", values=None):
+    from orbitquant_amd import ops
+
+    return ops.rotate_quantize(
+        xt.to(dev), torch.from_numpy(perm.astype(np.int32)).to(dev), torch.from_numpy(signs).to(dev),
+        torch.from_numpy(bounds).to(dev), block_size=block, eps=eps, inv_sqrt_block=float(inv),
+        centroids=None if cents is None else torch.from_numpy(cents).to(dev), code_format=fmt, values=values)
+
+
+# --------------------------------------------------------------- rotate+quantize
+
+RQ_CASES = [
+    # dim, block, a_bits, dtype, rows
+    (24, 8, 4, torch.float32, 7),
+    (37, 1, 4, torch.float32, 3),
+    (64, 64, 2, torch.bfloat16, 5),
+    (512, 512, 4, torch.bfloat16, 4),
+    (1152, 64, 4, torch.float32, 33),      # C1
+    (1152, 128, 4, torch.bfloat16, 40),    # C2 fc1
+    (4608, 512, 4, torch.bfloat16, 21),    # C2 fc2
+    (3072, 1024, 3, torch.bfloat16, 17),   # C3
+    (12288, 4096, 3, torch.bfloat16, 5),   # C3 fc2
+    (5120, 1024, 6, torch.bfloat16, 9),    # C4 fc1
+    (13824, 512, 6, torch.bfloat16, 5),    # C4 fc2
+    (4096, 4096, 4, torch.bfloat16, 16),   # C5
+    (14336, 2048, 4, torch.bfloat16, 4),   # C5 down
+    (16384, 16384, 4, torch.float16, 2),
+    (2048, 2, 8, torch.float16, 3),
+]
+
+
+@pytest.mark.parametrize(("dim", "block", "abits", "dtype", "rows"), RQ_CASES)
+def test_rotate_quantize_codes_and_norms_bit_exact(dev, dim, block, abits, dtype, rows):
+    rng = np.random.default_rng(dim * 31 + block)
+    perm, signs, block, inv = o.rpbh_constants(dim, 0, block)
+    cents, bounds = tables(max(dim, 3), abits)
+    xt, x32 = make_x(rng, rows, dim, dtype)
+    xt[rows // 2] = 0
+    x32[rows // 2] = 0
+    want_codes, want_norms = oracle_c.rotate_quantize(x32, perm, signs, bounds, block, 1e-10, inv)
+    codes, values, norms = gpu_rotate_quantize(dev, xt, perm, signs, bounds, block, 1e-10, inv, cents, "u8", "scaled")
+    assert np.array_equal(norms.cpu().numpy().view(np.int32), want_norms.view(np.int32))
+    got = codes.cpu().numpy()
+    mism = int((got != want_codes).sum())
+    assert mism == 0, f"{mism} code mismatches of {got.size}"
+    want_values = torch.from_numpy(cents[want_codes] * want_norms[:, None]).to(dtype)
+    assert torch.equal(values.cpu(), want_values)
+    assert not values[rows // 2].any()
+    if abits <= 4 and dim % 2 == 0:
+        nib, unit, norms2 = gpu_rotate_quantize(dev, xt, perm, signs, bounds, block, 1e-10, inv, cents, "nibble", "unit_bf16")
+        assert np.array_equal(nib.cpu().numpy(), o.pack_nibbles(want_codes))
+        assert torch.equal(norms2, norms)
+        assert torch.equal(unit.cpu(), torch.from_numpy(cents[want_codes]).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("dim", [512, 4096, 16384])
+def test_rotate_quantize_one_hot_rows(dev, dim):
+    # native tests/test_packed_matmul.py:688-733 (reference checkout): closed form per row
+    gen = torch.Generator().manual_seed(dim)
+    perm = torch.randperm(dim, generator=gen).numpy()
+    signs = np.where(np.arange(dim) % 2 == 0, 1, -1).astype(np.int8)
+    bounds = np.linspace(-0.2, 0.2, 15, dtype=F32)
+    x = torch.zeros((2, dim), dtype=torch.bfloat16)
+    x[0, 3] = 1
+    x[1, dim - 7] = -1
+    inv = F32(dim ** -0.5)
+    nib, _, norms = gpu_rotate_quantize(dev, x, perm, signs, bounds, dim, 1e-12, inv, None, "nibble")
+    assert norms.cpu().tolist() == [1.0, 1.0]
+    rows = []
+    for hot, val in ((3, 1.0), (dim - 7, -1.0)):
+        c = int(np.nonzero(perm == hot)[0][0])
+        j = np.arange(dim)
+        parity = np.array([bin(v).count("1") & 1 for v in (c & j)])
+        rot = (np.where(parity == 1, -1.0, 1.0) * val * signs[c]).astype(F32) * inv
+        rows.append(np.searchsorted(bounds, rot, side="left").astype(np.uint8))
+    assert np.array_equal(nib.cpu().numpy(), o.pack_nibbles(np.stack(rows)))
+
+
+def test_rotate_quantize_full_size_c2_bit_exact(dev):
+    # BASELINE config 2, second quantizer: [2048, 4608] bf16 with outlier columns x30
+    rng = np.random.default_rng(2)
+    m, dim = 2048, 4608
+    perm, signs, block, inv = o.rpbh_constants(dim, 0)
+    cents, bounds = tables(dim, 4)
+    x = rng.standard_normal((m, dim)).astype(F32)
+    x[:, rng.choice(dim, 23, replace=False)] *= 30
+    xt = torch.from_numpy(x).to(torch.bfloat16)
+    want_codes, want_norms = oracle_c.rotate_quantize(xt.float().numpy(), perm, signs, bounds, block, 1e-10, inv)
+    codes, _, norms = gpu_rotate_quantize(dev, xt, perm, signs, bounds, block, 1e-10, inv)
+    assert np.array_equal(norms.cpu().numpy().view(np.int32), want_norms.view(np.int32))
+    assert int((codes.cpu().numpy() != want_codes).sum()) == 0
+    # batch independence: any slice of rows gives the same codes
+    part, _, _ = gpu_rotate_quantize(dev, xt[100:117], perm, signs, bounds, block, 1e-10, inv)
+    assert torch.equal(part, codes[100:117])
+
+
+def test_rotate_quantize_rejects_bad_arguments(dev):
+    perm, signs, block, inv = o.rpbh_constants(64, 0, 64)
+    _, bounds = tables(64, 4)
+    x = torch.zeros((2, 64), dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        gpu_rotate_quantize(dev, x, perm, signs, bounds, 48, 1e-10, inv)       # not a power of two
+    _, b6 = tables(64, 6)
+    with pytest.raises(ValueError):
+        gpu_rotate_quantize(dev, x, perm, signs, b6, 64, 1e-10, inv, fmt="nibble")   # 64 levels in a nibble
+
+
+# ---------------------------------------------------------------------- unpack
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_unpack_lowbit_bit_exact(dev, bits):
+    from orbitquant_amd import ops
+
+    values = (np.arange(100003) * 7 % (1 << bits)).astype(np.uint8)
+    packed = o.pack_bits(values, bits)
+    got = ops.unpack_lowbit(torch.from_numpy(packed).to(dev), bits, values.size)
+    assert np.array_equal(got.cpu().numpy(), values)
+
+
+# ---------------------------------------------------------------- packed linear
+
+def make_layer(rng, n, k, wbits, abits, block="paper", scale=0.02, with_bias=True):
+    perm, signs, block, inv = o.rpbh_constants(k, 0, block)
+    cw, bw = tables(k, wbits)
+    ca, ba = tables(k, abits)
+    w = (rng.standard_normal((n, k)) * scale).astype(F32)
+    packed, r_bf16, idx = o.quantize_weight(w, perm, signs, bw, block, 1e-10, wbits)
+    bias = rng.standard_normal(n).astype(F32) * 0.1 if with_bias else None
+    return dict(perm=perm, signs=signs, block=block, inv=inv, cw=cw, bw=bw, ca=ca, ba=ba, packed=packed,
+                r=r_bf16, idx=idx, bias=bias, n=n, k=k, wbits=wbits, abits=abits)
+
+
+def check_outputs(got, want, s, r, k, what=""):
+    got = got.astype(np.float64)
+    bound = 2e-2 * s[:, None].astype(np.float64) * r[None, :].astype(np.float64) / math.sqrt(k)
+    err = np.abs(got - want)
+    # the output dtype's own rounding (bf16: 2^-9 relative) is not the kernel's error
+    slack = np.abs(want) * 2.0 ** -8 + 1e-30
+    worst = float((err / (bound + slack)).max())
+    assert worst <= 1.0, f"{what}: max error is {worst:.3f} of the bound"
+    cos = float((got * want).sum() / (np.linalg.norm(got) * np.linalg.norm(want) + 1e-300))
+    assert cos >= 0.9999, f"{what}: cosine {cos}"
+    return worst, cos
+
+
+def run_packed_linear(dev, layer, codes_np, s_np, fmt, out_dtype=torch.bfloat16):
+    from orbitquant_amd import ops
+
+    if fmt == "nibble":
+        codes_t = torch.from_numpy(o.pack_nibbles(codes_np))
+    else:
+        codes_t = torch.from_numpy(codes_np)
+    bias = None if layer["bias"] is None else torch.from_numpy(layer["bias"]).to(out_dtype).to(dev)
+    return ops.packed_linear(
+        codes_t.to(dev), torch.from_numpy(s_np).to(dev), torch.from_numpy(layer["ca"]).to(dev),
+        torch.from_numpy(layer["packed"]).to(dev), layer["r"].to(dev), torch.from_numpy(layer["cw"]).to(dev),
+        code_format=fmt, activation_bits=layer["abits"], weight_bits=layer["wbits"],
+        out_features=layer["n"], in_features=layer["k"], bias=bias, output_dtype=out_dtype)
+
+
+def oracle_linear(layer, codes, s, out_dtype):
+    bias = layer["bias"]
+    if bias is not None:
+        bias = torch.from_numpy(bias).to(out_dtype).float().numpy()
+    return oracle_c.linear_from_codes(codes, s, layer["ca"], layer["packed"], layer["wbits"],
+                                      layer["r"].float().numpy(), layer["cw"], bias, layer["n"])
+
+
+GEMM_CASES = [
+    # m, n, k, wbits, abits, block, bias, out dtype
+    (256, 1152, 1152, 4, 4, 64, True, torch.float32),      # C1 full size
+    (300, 200, 1152, 4, 4, "paper", True, torch.bfloat16), # ragged M and N
+    (130, 258, 256, 4, 4, "paper", False, torch.bfloat16),
+    (257, 384, 3072, 3, 3, "paper", True, torch.bfloat16), # C3 widths
+    (129, 96, 4608, 2, 4, "paper", True, torch.bfloat16),
+    (200, 160, 1024, 6, 4, "paper", False, torch.float16),
+    (100, 130, 512, 8, 4, "paper", True, torch.bfloat16),
+    (64, 64, 64, 4, 2, "paper", True, torch.bfloat16),
+    (33, 70, 192, 3, 4, "paper", True, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize(("m", "n", "k", "wbits", "abits", "block", "with_bias", "out_dtype"), GEMM_CASES)
+def test_packed_linear_tile_kernel(dev, m, n, k, wbits, abits, block, with_bias, out_dtype):
+    rng = np.random.default_rng(m * 7 + n * 3 + k + wbits)
+    layer = make_layer(rng, n, k, wbits, abits, block, with_bias=with_bias)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    x32[1] = 0
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, out_dtype)
+    got = run_packed_linear(dev, layer, codes, s, "nibble", out_dtype)
+    assert got.dtype == out_dtype and tuple(got.shape) == (m, n)
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "nibble")
+    # zero token -> exactly the bias (tests/test_paper_reference_oracle.py:202-203, reference checkout)
+    zero_row = got[1].float().cpu().numpy()
+    expect = np.zeros(n) if layer["bias"] is None else torch.from_numpy(layer["bias"]).to(out_dtype).float().numpy()
+    assert np.array_equal(zero_row, expect)
+    # one code per byte takes the shape-agnostic kernel: same answer
+    got_u8 = run_packed_linear(dev, layer, codes, s, "u8", out_dtype)
+    check_outputs(got_u8.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "u8")
+
+
+@pytest.mark.parametrize("tile", ["0", "1", "2"])
+def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
+    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+    rng = np.random.default_rng(int(tile) + 50)
+    m, n, k = 515, 520, 1152
+    layer = make_layer(rng, n, k, 4, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    got = run_packed_linear(dev, layer, codes, s, "nibble")
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, f"tile {tile}")
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 3])
+@pytest.mark.parametrize(("n", "k", "wbits"), [(4096, 4096, 2), (1000, 4096, 3), (4096, 14336, 3), (2048, 4096, 4), (512, 1152, 6), (256, 1024, 8)])
+def test_packed_linear_small_m_stream_kernel(dev, m, n, k, wbits):
+    rng = np.random.default_rng(m + n + k + wbits)
+    layer = make_layer(rng, n, k, wbits, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16, kind="plain")
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    got = run_packed_linear(dev, layer, codes, s, "nibble")
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "small-M")
+    again = run_packed_linear(dev, layer, codes, s, "nibble")
+    assert torch.equal(got, again)      # fixed summation order: run-to-run identical
+
+
+# ------------------------------------------------- float-activation packed matmul
+
+def _pack_loop(values, bits):
+    out = bytearray((len(values) * bits + 7) // 8)
+    for i, v in enumerate(values):
+        start = i * bits
+        out[start // 8] |= (v << (start % 8)) & 0xFF
+        if start % 8 + bits > 8:
+            out[start // 8 + 1] |= v >> (8 - start % 8)
+    return np.frombuffer(bytes(out), dtype=np.uint8).copy()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 6])
+@pytest.mark.parametrize(("rows", "k", "n"), [(9, 16, 7), (9, 19, 7), (15, 37, 29), (65, 64, 70), (1, 32, 32)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_matmul_packed_weight_reference_vectors(dev, bits, rows, k, n, dtype):
+    """Vectors of the reference's native tests (tests/test_packed_matmul.py:365-452,567-602 of
+    the native package): indices = arange % 2^b, centroids = linspace(-1, 1),
+    row_norms = linspace(0.5, 1.5), tolerance 2e-2 (3e-2 for bf16)."""
+    from orbitquant_amd import ops
+
+    torch.manual_seed(1000 + bits * 100 + rows * 10 + k + n)
+    x = torch.randn(rows, k).to(dtype)
+    idx = (np.arange(n * k) % (1 << bits)).astype(np.uint8)
+    packed = _pack_loop(idx.tolist(), bits)
+    r = torch.linspace(0.5, 1.5, n).to(torch.bfloat16)
+    cents = torch.linspace(-1.0, 1.0, 1 << bits)
+    bias = torch.randn(n).to(dtype)
+    w = r.float()[:, None] * cents[torch.from_numpy(idx.reshape(n, k)).long()]
+    want = torch.nn.functional.linear(x.float(), w, bias.float())
+    got = ops.matmul_packed_weight_values(
+        x.to(dev), torch.from_numpy(packed).to(dev), r.to(dev), cents.to(dev), bits=bits,
+        out_features=n, in_features=k, bias=bias.to(dev))
+    assert got.dtype == dtype and tuple(got.shape) == (rows, n)
+    tol = 3e-2 if dtype == torch.bfloat16 else 2e-2
+    assert torch.allclose(got.float().cpu(), want, atol=tol, rtol=tol)
+
+
+def test_matmul_packed_weight_mfma_path_realistic(dev):
+    from orbitquant_amd import ops
+
+    rng = np.random.default_rng(77)
+    m, n, k = 333, 1536, 1536
+    layer = make_layer(rng, n, k, 4, 4)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(F32)).to(torch.bfloat16)
+    got = ops.matmul_packed_weight_values(
+        x.to(dev), torch.from_numpy(layer["packed"]).to(dev), layer["r"].to(dev),
+        torch.from_numpy(layer["cw"]).to(dev), bits=4, out_features=n, in_features=k,
+        bias=torch.from_numpy(layer["bias"]).to(torch.bfloat16).to(dev))
+    bias = torch.from_numpy(layer["bias"]).to(torch.bfloat16).float().numpy()
+    want = o.matmul_packed_weight_f32(x.float().numpy(), layer["packed"], layer["r"].float().numpy(), layer["cw"], 4, n, bias)
+    s = np.linalg.norm(x.float().numpy(), axis=1)
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "float-activation MFMA")
+
+
+# ------------------------------------------------------------------ whole module
+
+@pytest.mark.parametrize(("name", "k", "n", "m", "dtype"), [
+    ("w4a4", 1152, 1152, 256, torch.float32),
+    ("w3a3", 3072, 512, 200, torch.bfloat16),
+    ("w2a4", 4096, 1024, 4, torch.bfloat16),
+    ("w2a3", 1024, 256, 40, torch.bfloat16),
+    ("w4a6", 5120, 384, 100, torch.bfloat16),
+])
+def test_orbit_linear_end_to_end(dev, name, k, n, m, dtype):
+    from orbitquant_amd import OrbitLinear, recipe
+
+    torch.manual_seed(5)
+    cfg = recipe(name)
+    lin = torch.nn.Linear(k, n)
+    with torch.no_grad():
+        lin.weight.mul_(0.6)
+    layer = OrbitLinear.from_linear(lin, config=cfg).to(dev)
+    assert sorted(layer.state_dict().keys()) == ["bias", "packed_weight_indices", "row_norms"]
+    x = torch.randn(2, m // 2, k).to(dtype)
+    x[0, 0] = 0
+    y = layer(x.to(dev))
+    assert y.dtype == dtype and tuple(y.shape) == (2, m // 2, n)
+
+    perm, signs, block, inv = o.rpbh_constants(k, 0)
+    ca, ba = tables(k, cfg.activation_bits)
+    cw, _ = tables(k, cfg.weight_bits)
+    x32 = x.reshape(-1, k).float().numpy()
+    codes, s = oracle_c.rotate_quantize(x32, perm, signs, ba, block, 1e-10, inv)
+    packed = layer.packed_weight_indices.cpu().numpy()
+    r = layer.row_norms.float().cpu().numpy()
+    bias = lin.bias.detach().to(dtype).float().numpy()
+    want = oracle_c.linear_from_codes(codes, s, ca, packed, cfg.weight_bits, r, cw, bias, n)
+    check_outputs(y.reshape(-1, n).float().cpu().numpy(), want, s, r, k, name)
+    assert np.array_equal(y[0, 0].float().cpu().numpy(), bias)
+
+    # the weights the module holds are the oracle's (offline quantization parity)
+    w_packed, w_r, _ = o.quantize_weight(lin.weight.detach().numpy(), perm, signs, tables(k, cfg.weight_bits)[1], block, 1e-10, cfg.weight_bits)
+    assert np.array_equal(packed, w_packed) and torch.equal(layer.row_norms.cpu(), w_r)
+
+
+def test_orbit_linear_torch_compile_fullgraph(dev):
+    # tests/test_torch_compile.py:30-90 of the reference: compiled == eager exactly
+    from orbitquant_amd import OrbitLinear, recipe
+
+    torch.manual_seed(9)
+    layer = OrbitLinear.from_linear(torch.nn.Linear(512, 256), config=recipe("w4a4")).to(dev)
+    x = torch.randn(3, 20, 512, dtype=torch.bfloat16, device=dev)
+    eager = layer(x)
+    compiled = torch.compile(layer, fullgraph=True)
+    assert torch.equal(compiled(x), eager)
+
+
+def test_state_dict_roundtrip(dev):
+    from orbitquant_amd import OrbitLinear, recipe
+
+    torch.manual_seed(3)
+    cfg = recipe("w3a3")
+    a = OrbitLinear.from_linear(torch.nn.Linear(256, 128), config=cfg).to(dev)
+    b = OrbitLinear.from_linear(torch.nn.Linear(256, 128), config=cfg).to(dev)
+    b.load_state_dict(a.state_dict(), strict=True)
+    x = torch.randn(17, 256, dtype=torch.bfloat16, device=dev)
+    assert torch.equal(a(x), b(x))
