@@ -7,9 +7,10 @@ exception is raised.
 from __future__ import annotations
 
 import ctypes
+import os
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "liborbitquant_hip.so"
+LIB_PATH = Path(os.environ.get("ORBITQUANT_HIP_LIB") or Path(__file__).resolve().parent / "liborbitquant_hip.so")
 
 OQ_F32, OQ_F16, OQ_BF16 = 0, 1, 2
 OQ_CODES_U8, OQ_CODES_NIBBLE = 0, 1

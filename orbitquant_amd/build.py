@@ -9,6 +9,7 @@ algorithm bit for bit); packed fp32 VALU instructions are disabled everywhere.
 
 from __future__ import annotations
 
+import os
 import subprocess
 import sys
 import time
@@ -30,6 +31,8 @@ SOURCES = {
     "rotate_quantize.hip": ["-ffp-contract=off"],
     "packed_generic.hip": [],
     "packed_gemm.hip": [],
+    "packed_gemm_staged.hip": [],
+    "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
 }
 
@@ -44,7 +47,7 @@ def _compile(item) -> Path:
         newest = max(p.stat().st_mtime for p in list(CSRC.glob("*.h")) + [CSRC / name, PKG.parent / "include/orbitquant_hip.h"])
         if obj.stat().st_mtime > newest:
             return obj
-    cmd = COMMON + extra + ["-c", str(CSRC / name), "-o", str(obj)]
+    cmd = COMMON + extra + os.environ.get("OQ_HIPCC_FLAGS", "").split() + ["-c", str(CSRC / name), "-o", str(obj)]
     t0 = time.time()
     proc = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
     noise = "'-packed-fp32-ops' is not a recognized feature for this target"  # host pass only

@@ -20,12 +20,9 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
 
-// round-to-nearest-even fp32 -> bf16 bits (NaN kept quiet)
+// round-to-nearest-even fp32 -> bf16 bits (the gfx950 conversion instruction)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {

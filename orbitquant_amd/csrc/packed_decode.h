@@ -1,5 +1,17 @@
 // Lookup-table decode of packed low-bit indices into 16-bit MFMA operands,
 // shared by the tiled GEMM and the small-M streaming kernel.
+//
+// Every table lives in LDS and is replicated 32 times: entry e occupies 128
+// bytes, copy c of it sits at byte e*128 + c*4, and lane l always reads copy
+// l%32.  A wavefront therefore never presents two different addresses to one
+// LDS bank, whatever indices its lanes hold.  A lookup costs two VALU
+// instructions (bit-field extract, shift-add of the lane's base) and one
+// ds_read_b32.
+//
+//   widths 2, 3, 4 : the table is indexed by a PAIR of codes (2*bits bits) and
+//                    returns both 16-bit values in one dword
+//   widths 6, 8    : one code per lookup; the entry holds the value in both
+//                    halves so two lookups merge with one bit-select
 #pragma once
 
 #include "oq_common.h"
@@ -9,52 +21,73 @@ namespace oq {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// ---- lookup-table geometry ---------------------------------------------------
+typedef __attribute__((address_space(3))) const uint32_t lds_cu32;
+
+#if defined(__HIP_DEVICE_COMPILE__)
+__device__ __forceinline__ uint32_t lds_read_u32(uint32_t byte_addr) { return *(lds_cu32 *)(byte_addr); }
+
+__device__ __forceinline__ uint32_t lds_byte_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+#else  // the host pass only needs the declarations to parse
+__device__ uint32_t lds_read_u32(uint32_t byte_addr);
+__device__ uint32_t lds_byte_address(const void *p);
+#endif
+
 template <int BITS> struct WLut {
-  static constexpr int kPairBits = BITS == 8 ? 8 : 2 * BITS;      // 8-bit: single-code table
-  static constexpr int kEntries = 1 << kPairBits;
-  static constexpr int kLogRep = kEntries <= 256 ? 5 : 0;        // replicate small tables x32
-  static constexpr int kDwords = kEntries << kLogRep;
+  static constexpr bool kPair = BITS <= 4;
+  static constexpr int kIndexBits = kPair ? 2 * BITS : BITS;
+  static constexpr int kEntries = 1 << kIndexBits;
+  static constexpr int kDwords = kEntries * 32;  // 128 bytes per entry
 };
-constexpr int kALutLogRep = 5;
-constexpr int kALutDwords = 256 << kALutLogRep;
+constexpr int kALutDwords = 256 * 32;  // pair table of 4-bit activation codes
 
-__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
-  return static_cast<uint32_t>(f32_to_bf16_bits(lo)) | (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
-}
-__device__ __forceinline__ uint32_t f16_pair(float lo, float hi) {
-  return static_cast<uint32_t>(f32_to_f16_bits(lo)) | (static_cast<uint32_t>(f32_to_f16_bits(hi)) << 16);
+__device__ __forceinline__ uint32_t pack16(float lo, float hi, bool f16) {
+  const uint32_t a = f16 ? f32_to_f16_bits(lo) : f32_to_bf16_bits(lo);
+  const uint32_t b = f16 ? f32_to_f16_bits(hi) : f32_to_bf16_bits(hi);
+  return a | (b << 16);
 }
 
-// Fill a (possibly replicated) pair table: entry p holds (c[p & mask], c[p >> bits]).
-template <bool F16>
-__device__ __forceinline__ void fill_pair_lut(uint32_t *lut, const float *cents, int bits, int levels,
-                                              int pair_bits, int log_rep, bool single) {
-  const int total = (1 << pair_bits) << log_rep;
+// Fill a replicated table.  pair: entry e = (c[e & mask], c[e >> bits]); single: (c[e], c[e]).
+__device__ __forceinline__ void fill_lut(uint32_t *lut, const float *cents, int bits, int levels, bool pair,
+                                         bool f16) {
+  const int entries = 1 << (pair ? 2 * bits : bits);
   const int mask = (1 << bits) - 1;
-  for (int i = threadIdx.x; i < total; i += blockDim.x) {
-    const int p = i >> log_rep;
-    const int c0 = p & mask, c1 = single ? 0 : (p >> bits);
+  for (int e = threadIdx.x; e < entries; e += blockDim.x) {
+    const int c0 = pair ? (e & mask) : e;
+    const int c1 = pair ? (e >> bits) : e;
     const float v0 = c0 < levels ? cents[c0] : 0.0f;
-    const float v1 = (!single && c1 < levels) ? cents[c1] : 0.0f;
-    lut[i] = F16 ? f16_pair(v0, v1) : bf16_pair(v0, v1);
+    const float v1 = c1 < levels ? cents[c1] : 0.0f;
+    const uint32_t d = pack16(v0, v1, f16);
+    uint4 *dst = reinterpret_cast<uint4 *>(lut + e * 32);
+    const uint4 v = make_uint4(d, d, d, d);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = v;
   }
 }
 
-// ---- weight decode: dwords of one lane's 32-value run -> operand of MFMA q ------
+// `base` = LDS byte address of the table + 4 * (lane % 32)
+__device__ __forceinline__ uint32_t lut_at(uint32_t base, uint32_t index) { return lds_read_u32((index << 7) + base); }
+
+// table lookup of the `width`-bit field of `word` at bit `pos` (both compile-time after unrolling)
+__device__ __forceinline__ uint32_t lut_field(uint32_t base, uint32_t word, int pos, int width) {
+  return lds_read_u32((__builtin_amdgcn_ubfe(word, pos, width) << 7) + base);
+}
+
+// ---- weight decode: the dwords of one lane's 32-value run -> operand of MFMA q ----
 template <int BITS>
-__device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, const uint32_t *lut, int rl) {
-  constexpr int LR = WLut<BITS>::kLogRep;
+__device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint32_t base) {
   uint32_t o[4];
   if constexpr (BITS == 4) {
     const uint32_t f = w[q];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut[(((f >> (8 * p)) & 0xffu) << LR) + rl];
+    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 8 * p, 8);
   } else if constexpr (BITS == 2) {
-    const uint32_t f = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
+    const uint32_t f = w[q >> 1] >> (16 * (q & 1));
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut[(((f >> (4 * p)) & 0xfu) << LR) + rl];
+    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 4 * p, 4);
   } else if constexpr (BITS == 3) {
     uint32_t f;
     if (q == 0) f = w[0];
@@ -62,33 +95,38 @@ __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, cons
     else if (q == 2) f = __builtin_amdgcn_alignbit(w[2], w[1], 16);
     else f = w[2] >> 8;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut[(((f >> (6 * p)) & 0x3fu) << LR) + rl];
+    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 6 * p, 6);
   } else if constexpr (BITS == 6) {
-    // 48-bit field at bit 48q of six dwords
-    uint64_t f;
-    if (q == 0) f = static_cast<uint64_t>(w[0]) | (static_cast<uint64_t>(w[1]) << 32);
-    else if (q == 1) f = static_cast<uint64_t>(w[1] >> 16) | (static_cast<uint64_t>(w[2]) << 16);
-    else if (q == 2) f = static_cast<uint64_t>(w[3]) | (static_cast<uint64_t>(w[4]) << 32);
-    else f = static_cast<uint64_t>(w[4] >> 16) | (static_cast<uint64_t>(w[5]) << 16);
+    // 48-bit field at bit 48q of six dwords: eight 6-bit codes
+    uint32_t lo, hi;  // lo: codes 0..4 and two bits of code 5; hi: the rest
+    if (q == 0) { lo = w[0]; hi = w[1]; }
+    else if (q == 1) { lo = __builtin_amdgcn_alignbit(w[2], w[1], 16); hi = w[2] >> 16; }
+    else if (q == 2) { lo = w[3]; hi = w[4]; }
+    else { lo = __builtin_amdgcn_alignbit(w[5], w[4], 16); hi = w[5] >> 16; }
+    const uint32_t mid = __builtin_amdgcn_alignbit(hi, lo, 24);  // bits 24..55 of the field
+    const uint32_t c[8] = {lo & 63u, (lo >> 6) & 63u, (lo >> 12) & 63u, (lo >> 18) & 63u,
+                           mid & 63u, (mid >> 6) & 63u, (mid >> 12) & 63u, (mid >> 18) & 63u};
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut[static_cast<uint32_t>(f >> (12 * p)) & 0xfffu];
-  } else {  // 8 bits: one code per table entry (value in the low half)
+    for (int p = 0; p < 4; ++p)
+      o[p] = __builtin_amdgcn_perm(lut_at(base, c[2 * p + 1]), lut_at(base, c[2 * p]), 0x07060100u);
+  } else {  // 8 bits
     const uint32_t lo = w[2 * q], hi = w[2 * q + 1];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const uint32_t src = p < 2 ? lo : hi;
-      const uint32_t e0 = lut[(((src >> (16 * (p & 1))) & 0xffu) << LR) + rl] & 0xffffu;
-      const uint32_t e1 = lut[(((src >> (16 * (p & 1) + 8)) & 0xffu) << LR) + rl] << 16;
-      o[p] = e0 | e1;
+      const uint32_t e0 = lut_at(base, (src >> (16 * (p & 1))) & 0xffu);
+      const uint32_t e1 = lut_at(base, (src >> (16 * (p & 1) + 8)) & 0xffu);
+      o[p] = __builtin_amdgcn_perm(e1, e0, 0x07060100u);
     }
   }
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-__device__ __forceinline__ uint4 decode_a_nibble(uint32_t f, const uint32_t *lut, int rl) {
+// eight 4-bit activation codes (one dword) -> operand of one MFMA
+__device__ __forceinline__ uint4 decode_a_nibble(uint32_t f, uint32_t base) {
   uint32_t o[4];
 #pragma unroll
-  for (int p = 0; p < 4; ++p) o[p] = lut[(((f >> (8 * p)) & 0xffu) << kALutLogRep) + rl];
+  for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 8 * p, 8);
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
@@ -109,6 +147,5 @@ __device__ __forceinline__ void load_w(const uint8_t *p, uint32_t (&w)[BITS]) {
     for (int i = 0; i < BITS; ++i) w[i] = d[i];
   }
 }
-
 
 }  // namespace oq

@@ -17,11 +17,8 @@
 // which makes every global load of packed data one contiguous 4*bits-byte run
 // per lane (16 bytes for 4-bit), with no cross-lane shuffles and no LDS staging.
 //
-// Lookup tables.  Two codes are decoded per LDS read: the table is indexed by
-// the 2*bits-bit pair and returns both bf16 values in one dword.  Tables of up
-// to 256 pairs are replicated 32 times so that lane l reads copy l%32 and a
-// wavefront never has two different addresses in one LDS bank.
-#include "packed_decode.h"
+// Lookup tables: see packed_decode.h (pair tables, replicated per LDS bank).
+#include "gemm_epilogue.h"
 
 namespace oq {
 namespace {
@@ -68,8 +65,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   uint32_t *wlut = lds;
   uint32_t *alut = lds + WLut<BITS>::kDwords;
 
-  fill_pair_lut<AM == A_F16>(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPairBits, WLut<BITS>::kLogRep, BITS == 8);
-  if constexpr (AM == A_NIBBLE) fill_pair_lut<false>(alut, g.act_cents, 4, g.a_levels, 8, kALutLogRep, false);
+  fill_lut(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPair, AM == A_F16);
+  if constexpr (AM == A_NIBBLE) fill_lut(alut, g.act_cents, 4, g.a_levels, true, false);
   __syncthreads();
 
   constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
@@ -87,7 +84,9 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int pid_n = (bid % width) / gsz;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, grp = lane >> 5, rl = lane & 31;
+  const int r = lane & 31, grp = lane >> 5;
+  const uint32_t wbase = lds_byte_address(wlut) + 4 * r;
+  const uint32_t abase = lds_byte_address(alut) + 4 * r;
   const int64_t m_base = static_cast<int64_t>(pid_m) * TM + (wave >> 1) * (FM * 32);
   const int64_t n_base = static_cast<int64_t>(pid_n) * TN + (wave & 1) * (FN * 32);
 
@@ -117,73 +116,89 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  ARaw<AM> a_nxt[FM];
-  uint32_t w_nxt[FN][BITS];
+  // ---- main loop: software pipeline over "q-steps" (one MFMA k-slice of 16) -------
+  // While the matrix core works on the operands decoded for q-step t, the wavefront
+  // issues the table lookups for q-step t+1; packed dwords for K-step ks+1 are in
+  // flight from global memory during K-step ks.
+  ARaw<AM> a_cur[FM], a_nxt[FM];
+  uint32_t w_cur[FN][BITS], w_nxt[FN][BITS];
 #pragma unroll
-  for (int i = 0; i < FM; ++i) load_a<AM>(ap[i], a_nxt[i]);
+  for (int i = 0; i < FM; ++i) load_a<AM>(ap[i], a_cur[i]);
 #pragma unroll
-  for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j], w_nxt[j]);
+  for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j], w_cur[j]);
 
   const int steps = static_cast<int>(g.K / 64);
+  if (steps > 1) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + A_ROW_STEP, a_nxt[i]);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + 8 * BITS, w_nxt[j]);
+  }
+
+  auto decode = [&](int q, uint4 (&af)[FM], uint4 (&bf)[FN]) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      if constexpr (AM == A_NIBBLE) {
+        const uint32_t f = q == 0 ? a_cur[i].v[0].x : q == 1 ? a_cur[i].v[0].y : q == 2 ? a_cur[i].v[0].z : a_cur[i].v[0].w;
+        af[i] = decode_a_nibble(f, abase);
+      } else {
+        af[i] = a_cur[i].v[q];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) bf[j] = decode_w<BITS>(w_cur[j], q, wbase);
+  };
+  auto multiply = [&](const uint4 (&af)[FM], const uint4 (&bf)[FN]) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(af[i], bf[j], acc[i][j]);
+  };
+  // interleave hint: after each MFMA, the lookups' address arithmetic and LDS reads
+  constexpr int kLookupsPerMfma = (AM == A_NIBBLE ? (FM + FN) : FN) * 4 / (FM * FN);
+  auto interleave = [&]() {
+#if defined(OQ_SCHED_HINTS)
+#pragma unroll
+    for (int i = 0; i < FM * FN; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2 * kLookupsPerMfma, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, kLookupsPerMfma, 0);
+    }
+#endif
+  };
+
+  uint4 af0[FM], bf0[FN], af1[FM], bf1[FN];
+  decode(0, af0, bf0);
   for (int ks = 0; ks < steps; ++ks) {
-    ARaw<AM> a_cur[FM];
-    uint32_t w_cur[FN][BITS];
+    decode(1, af1, bf1);
+    multiply(af0, bf0);
+    interleave();
+    decode(2, af0, bf0);
+    multiply(af1, bf1);
+    interleave();
+    decode(3, af1, bf1);
+    multiply(af0, bf0);
+    interleave();
+    // rotate: K-step ks+1 becomes current, K-step ks+2 goes in flight
 #pragma unroll
     for (int i = 0; i < FM; ++i) a_cur[i] = a_nxt[i];
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int d = 0; d < BITS; ++d) w_cur[j][d] = w_nxt[j][d];
-    if (ks + 1 < steps) {
+    if (ks + 2 < steps) {
 #pragma unroll
-      for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + static_cast<int64_t>(ks + 1) * A_ROW_STEP, a_nxt[i]);
+      for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + static_cast<int64_t>(ks + 2) * A_ROW_STEP, a_nxt[i]);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(ks + 1) * (8 * BITS), w_nxt[j]);
+      for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(ks + 2) * (8 * BITS), w_nxt[j]);
     }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      uint4 af[FM], bf[FN];
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        if constexpr (AM == A_NIBBLE) {
-          const uint32_t f = q == 0 ? a_cur[i].v[0].x : q == 1 ? a_cur[i].v[0].y : q == 2 ? a_cur[i].v[0].z : a_cur[i].v[0].w;
-          af[i] = decode_a_nibble(f, alut, rl);
-        } else {
-          af[i] = a_cur[i].v[q];
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < FN; ++j) bf[j] = decode_w<BITS>(w_cur[j], q, wlut, rl);
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(af[i], bf[j], acc[i][j]);
-    }
+    decode(0, af0, bf0);  // of K-step ks+1 (unused after the last step)
+    multiply(af1, bf1);
+    interleave();
   }
 
-  // ---- epilogue: acc * scale[m] * r_w[n] + bias[n] ------------------------------
-  // accumulator e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32 of its 32x32 tile
-#pragma unroll
-  for (int j = 0; j < FN; ++j) {
-    const int64_t n = n_base + 32 * j + r;
-    if (n >= g.N) continue;
-    const float rn = bf16_bits_to_f32(g.row_norms[n]);
-    const float bv = g.bias != nullptr ? load_dyn_f32(g.bias, g.bias_dtype, n) : 0.0f;
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int64_t m = m_base + 32 * i + 8 * (e >> 2) + 4 * grp + (e & 3);
-        if (m >= g.M) continue;
-        const float sc = g.row_scale != nullptr ? g.row_scale[m] : 1.0f;
-        const float y = acc[i][j][e] * sc * rn + bv;
-        const int64_t o = m * g.N + n;
-        if (g.out_dtype == OQ_BF16) static_cast<uint16_t *>(g.out)[o] = f32_to_bf16_bits(y);
-        else if (g.out_dtype == OQ_F16) static_cast<uint16_t *>(g.out)[o] = f32_to_f16_bits(y);
-        else static_cast<float *>(g.out)[o] = y;
-      }
-    }
-  }
+  gemm_epilogue<FM, FN>(acc, m_base, n_base, r, grp, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.out,
+                        g.out_dtype);
 }
 
 template <int AM, int BITS, int FM, int FN>
@@ -223,8 +238,10 @@ int launch_mode(const GemmArgs &g, int bits, int tile, hipStream_t stream) {
   }
 }
 
+}  // namespace
+
 // Tile choice: the largest tile that still gives every CU work.
-int choose_tile(int64_t M, int64_t N) {
+int gemm_choose_tile(int64_t M, int64_t N) {
   const char *force = getenv("OQ_GEMM_TILE");
   if (force != nullptr && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
   auto tiles = [&](int tm, int tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
@@ -232,8 +249,6 @@ int choose_tile(int64_t M, int64_t N) {
   if (tiles(128, 256) >= 384) return 1;
   return 0;
 }
-
-}  // namespace
 
 bool gemm_supported(int64_t K, int bits) {
   return K % 64 == 0 && (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
@@ -248,13 +263,9 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
-  const int tile = choose_tile(M, N);
-  switch (a_mode) {
-    case A_NIBBLE: return launch_mode<A_NIBBLE>(g, bits, tile, stream);
-    case A_BF16: return launch_mode<A_BF16>(g, bits, tile, stream);
-    case A_F16: return launch_mode<A_F16>(g, bits, tile, stream);
-    default: return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
-  }
+  const int tile = gemm_choose_tile(M, N);
+  if (a_mode != A_NIBBLE) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
+  return launch_mode<A_NIBBLE>(g, bits, tile, stream);
 }
 
 }  // namespace oq

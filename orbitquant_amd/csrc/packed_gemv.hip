@@ -17,8 +17,6 @@
 namespace oq {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
 struct GemvArgs {
   const uint8_t *a;          // nibble codes [M, K/2]
   const float *row_scale;    // [M] or NULL
@@ -42,12 +40,14 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   uint32_t *alut = lds + WLut<BITS>::kDwords;
   float *partial = reinterpret_cast<float *>(alut + kALutDwords);  // [WAVES][R][64][4]
 
-  fill_pair_lut<false>(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPairBits, WLut<BITS>::kLogRep, BITS == 8);
-  fill_pair_lut<false>(alut, g.act_cents, 4, g.a_levels, 8, kALutLogRep, false);
+  fill_lut(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPair, false);
+  fill_lut(alut, g.act_cents, 4, g.a_levels, true, false);
   __syncthreads();
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, grp = lane >> 4, rl = lane & 31;
+  const int r = lane & 15, grp = lane >> 4;
+  const uint32_t wbase = lds_byte_address(wlut) + 4 * (lane & 31);
+  const uint32_t abase = lds_byte_address(alut) + 4 * (lane & 31);
   const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * R);
 
   const int steps = static_cast<int>(g.K / 128);
@@ -89,10 +89,10 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const uint32_t f = q == 0 ? a_cur.x : q == 1 ? a_cur.y : q == 2 ? a_cur.z : a_cur.w;
-      const uint4 af = decode_a_nibble(f, alut, rl);
+      const uint4 af = decode_a_nibble(f, abase);
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        const uint4 bf = decode_w<BITS>(w_cur[j], q, wlut, rl);
+        const uint4 bf = decode_w<BITS>(w_cur[j], q, wbase);
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af), __builtin_bit_cast(bf16x8, bf),
                                                          acc[j], 0, 0, 0);
       }
