@@ -398,3 +398,70 @@ def test_state_dict_roundtrip(dev):
     b.load_state_dict(a.state_dict(), strict=True)
     x = torch.randn(17, 256, dtype=torch.bfloat16, device=dev)
     assert torch.equal(a(x), b(x))
+
+
+# -------------------------------------------- drop-in package (reference API names)
+
+@pytest.mark.parametrize(("dim", "threads"), [(512, 128), (4096, 256), (16384, 512)])
+def test_dropin_quantize_activations_packed_w4_and_int8(dev, dim, threads):
+    """Reference native tests (tests/test_packed_matmul.py:773-821 of the native package):
+    the int8 form equals codes[index] of the packed form, norms identical."""
+    import orbitquant_packed_matmul as pkg
+
+    torch.manual_seed(dim)
+    x = torch.randn((2, dim), dtype=torch.bfloat16)
+    perm = torch.randperm(dim)
+    signs = torch.where(torch.arange(dim) % 2 == 0, 1, -1).to(torch.int8)
+    bounds = torch.linspace(-0.2, 0.2, 15)
+    codes = torch.tensor([-120, -92, -68, -49, -34, -22, -12, -4, 4, 12, 22, 34, 49, 68, 92, 120], dtype=torch.int8)
+    kw = dict(eps=1e-12, inv_sqrt_block=dim ** -0.5, threads=threads)
+    packed, norms = pkg.quantize_activations_packed_w4(x.to(dev), perm.to(dev), signs.to(dev), bounds.to(dev), **kw)
+    q8, norms8 = pkg.quantize_activations_int8(x.to(dev), perm.to(dev), signs.to(dev), bounds.to(dev), codes.to(dev), **kw)
+    assert packed.dtype == torch.uint8 and tuple(packed.shape) == (2, dim // 2) and tuple(norms.shape) == (2,)
+    idx = torch.empty((2, dim), dtype=torch.long, device=dev)
+    idx[:, 0::2] = packed & 15
+    idx[:, 1::2] = packed >> 4
+    assert torch.equal(q8, codes.to(dev)[idx]) and torch.equal(norms8, norms)
+    want_codes, want_norms = oracle_c.rotate_quantize(x.float().numpy(), perm.numpy(), signs.numpy(), bounds.numpy(), dim, 1e-12, F32(dim ** -0.5))
+    assert np.array_equal(packed.cpu().numpy(), o.pack_nibbles(want_codes))
+    assert np.array_equal(norms.cpu().numpy(), want_norms)
+    # int32 and int64 permutations give the same result (tests/test_packed_matmul.py:736-770)
+    packed32, _ = pkg.quantize_activations_packed_w4(x.to(dev), perm.to(torch.int32).to(dev), signs.to(dev), bounds.to(dev), **kw)
+    assert torch.equal(packed32, packed)
+
+
+@pytest.mark.parametrize(("rows", "out_features"), [(128, 128), (256, 128), (130, 258)])
+def test_dropin_matmul_packed_w4a4_int8_exact_integer_reference(dev, rows, out_features):
+    # reference native tests/test_packed_matmul.py:605-685: fixed int8 code table, scales 0.005
+    import orbitquant_packed_matmul as pkg
+
+    k = 256
+    torch.manual_seed(0)
+    a_idx = torch.randint(0, 16, (rows, k), dtype=torch.uint8)
+    w_idx = torch.randint(0, 16, (out_features, k), dtype=torch.uint8)
+    pa = (a_idx[:, 0::2] | (a_idx[:, 1::2] << 4)).contiguous()
+    pw = (w_idx[:, 0::2] | (w_idx[:, 1::2] << 4)).contiguous()
+    codes = torch.tensor([-104, -79, -62, -48, -36, -25, -15, -5, 5, 15, 25, 36, 48, 62, 79, 104], dtype=torch.int8)
+    tn = torch.linspace(0.5, 1.0, rows)
+    rn = torch.linspace(0.5, 1.5, out_features).to(torch.bfloat16)
+    got = pkg.matmul_packed_w4a4_int8(pa.to(dev), pw.to(dev), tn.to(dev), rn.to(dev), codes.to(dev), codes.to(dev),
+                                      activation_scale=0.005, weight_scale=0.005, out_features=out_features, in_features=k)
+    ref = codes[a_idx.long()].float() @ codes[w_idx.long()].float().T
+    ref = ref * tn[:, None] * rn.float()[None, :] * (0.005 * 0.005)
+    assert got.dtype == torch.bfloat16
+    assert torch.allclose(got.float().cpu(), ref, atol=0.25, rtol=1e-2)
+
+
+def test_dropin_matmul_packed_weight_rows_1536(dev):
+    # reference native tests/test_packed_matmul.py:222-279: realistic 1536 rows 16/24/32/33
+    import orbitquant_packed_matmul as pkg
+
+    rng = np.random.default_rng(1536)
+    layer = make_layer(rng, 1536, 1536, 4, 4)
+    for rows in (16, 24, 32, 33):
+        x = torch.from_numpy(rng.standard_normal((rows, 1536)).astype(F32)).to(torch.bfloat16)
+        got = pkg.matmul_packed_weight(x.to(dev), torch.from_numpy(layer["packed"]), layer["r"], torch.from_numpy(layer["cw"]),
+                                       bits=4, out_features=1536, in_features=1536)
+        want = o.matmul_packed_weight_f32(x.float().numpy(), layer["packed"], layer["r"].float().numpy(), layer["cw"], 4, 1536)
+        s = np.linalg.norm(x.float().numpy(), axis=1)
+        check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), 1536, f"rows {rows}")
