@@ -36,13 +36,16 @@ __device__ uint32_t lds_read_u32(uint32_t byte_addr);
 __device__ uint32_t lds_byte_address(const void *p);
 #endif
 
-template <int BITS> struct WLut {
+// LR = log2(copies per entry): 5 for the MFMA-bound GEMM (no bank conflicts at all), 3 for the
+// HBM-bound small-M kernel (smaller tables, more workgroups per CU, a few 2-way conflicts).
+template <int BITS, int LR = 5> struct WLut {
   static constexpr bool kPair = BITS <= 4;
   static constexpr int kIndexBits = kPair ? 2 * BITS : BITS;
   static constexpr int kEntries = 1 << kIndexBits;
-  static constexpr int kDwords = kEntries * 32;  // 128 bytes per entry
+  static constexpr int kDwords = kEntries << LR;
 };
-constexpr int kALutDwords = 256 * 32;  // pair table of 4-bit activation codes
+constexpr int kALutDwords = 256 * 32;  // pair table of 4-bit activation codes, 32 copies
+template <int LR> constexpr int alut_dwords() { return 256 << LR; }
 
 __device__ __forceinline__ uint32_t pack16(float lo, float hi, bool f16) {
   const uint32_t a = f16 ? f32_to_f16_bits(lo) : f32_to_bf16_bits(lo);
@@ -51,6 +54,7 @@ __device__ __forceinline__ uint32_t pack16(float lo, float hi, bool f16) {
 }
 
 // Fill a replicated table.  pair: entry e = (c[e & mask], c[e >> bits]); single: (c[e], c[e]).
+template <int LR = 5>
 __device__ __forceinline__ void fill_lut(uint32_t *lut, const float *cents, int bits, int levels, bool pair,
                                          bool f16) {
   const int entries = 1 << (pair ? 2 * bits : bits);
@@ -61,33 +65,35 @@ __device__ __forceinline__ void fill_lut(uint32_t *lut, const float *cents, int 
     const float v0 = c0 < levels ? cents[c0] : 0.0f;
     const float v1 = c1 < levels ? cents[c1] : 0.0f;
     const uint32_t d = pack16(v0, v1, f16);
-    uint4 *dst = reinterpret_cast<uint4 *>(lut + e * 32);
+    uint4 *dst = reinterpret_cast<uint4 *>(lut + (e << LR));
     const uint4 v = make_uint4(d, d, d, d);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dst[i] = v;
+    for (int i = 0; i < (1 << LR) / 4; ++i) dst[i] = v;
   }
 }
 
-// `base` = LDS byte address of the table + 4 * (lane % 32)
-__device__ __forceinline__ uint32_t lut_at(uint32_t base, uint32_t index) { return lds_read_u32((index << 7) + base); }
+// `base` = LDS byte address of the table + 4 * (lane % copies)
+template <int LR = 5>
+__device__ __forceinline__ uint32_t lut_at(uint32_t base, uint32_t index) { return lds_read_u32((index << (LR + 2)) + base); }
 
 // table lookup of the `width`-bit field of `word` at bit `pos` (both compile-time after unrolling)
+template <int LR = 5>
 __device__ __forceinline__ uint32_t lut_field(uint32_t base, uint32_t word, int pos, int width) {
-  return lds_read_u32((__builtin_amdgcn_ubfe(word, pos, width) << 7) + base);
+  return lds_read_u32((__builtin_amdgcn_ubfe(word, pos, width) << (LR + 2)) + base);
 }
 
 // ---- weight decode: the dwords of one lane's 32-value run -> operand of MFMA q ----
-template <int BITS>
+template <int BITS, int LR = 5>
 __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint32_t base) {
   uint32_t o[4];
   if constexpr (BITS == 4) {
     const uint32_t f = w[q];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 8 * p, 8);
+    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 8 * p, 8);
   } else if constexpr (BITS == 2) {
     const uint32_t f = w[q >> 1] >> (16 * (q & 1));
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 4 * p, 4);
+    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 4 * p, 4);
   } else if constexpr (BITS == 3) {
     uint32_t f;
     if (q == 0) f = w[0];
@@ -95,7 +101,7 @@ __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint
     else if (q == 2) f = __builtin_amdgcn_alignbit(w[2], w[1], 16);
     else f = w[2] >> 8;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 6 * p, 6);
+    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 6 * p, 6);
   } else if constexpr (BITS == 6) {
     // 48-bit field at bit 48q of six dwords: eight 6-bit codes
     uint32_t lo, hi;  // lo: codes 0..4 and two bits of code 5; hi: the rest
@@ -108,14 +114,14 @@ __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint
                            mid & 63u, (mid >> 6) & 63u, (mid >> 12) & 63u, (mid >> 18) & 63u};
 #pragma unroll
     for (int p = 0; p < 4; ++p)
-      o[p] = __builtin_amdgcn_perm(lut_at(base, c[2 * p + 1]), lut_at(base, c[2 * p]), 0x07060100u);
+      o[p] = __builtin_amdgcn_perm(lut_at<LR>(base, c[2 * p + 1]), lut_at<LR>(base, c[2 * p]), 0x07060100u);
   } else {  // 8 bits
     const uint32_t lo = w[2 * q], hi = w[2 * q + 1];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const uint32_t src = p < 2 ? lo : hi;
-      const uint32_t e0 = lut_at(base, (src >> (16 * (p & 1))) & 0xffu);
-      const uint32_t e1 = lut_at(base, (src >> (16 * (p & 1) + 8)) & 0xffu);
+      const uint32_t e0 = lut_at<LR>(base, (src >> (16 * (p & 1))) & 0xffu);
+      const uint32_t e1 = lut_at<LR>(base, (src >> (16 * (p & 1) + 8)) & 0xffu);
       o[p] = __builtin_amdgcn_perm(e1, e0, 0x07060100u);
     }
   }
@@ -123,10 +129,11 @@ __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint
 }
 
 // eight 4-bit activation codes (one dword) -> operand of one MFMA
+template <int LR = 5>
 __device__ __forceinline__ uint4 decode_a_nibble(uint32_t f, uint32_t base) {
   uint32_t o[4];
 #pragma unroll
-  for (int p = 0; p < 4; ++p) o[p] = lut_field(base, f, 8 * p, 8);
+  for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 8 * p, 8);
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 

@@ -12,6 +12,9 @@
 // K is cut like in the tiled GEMM: in a K-step of 128, lane group g (0..3) owns
 // the contiguous run k0+32g .. k0+32g+31 of its row and MFMA q (0..3) consumes
 // values 8q..8q+7 of every run.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include "packed_decode.h"
 
 namespace oq {
@@ -33,21 +36,20 @@ struct GemvArgs {
   int out_dtype;
 };
 
+constexpr int kLR = 3;     // 8 copies per table entry
+constexpr int kDepth = 2;  // K-steps of 128 fetched per batch of global loads (two batches in flight)
+
 template <int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   extern __shared__ __align__(16) uint32_t lds[];
   uint32_t *wlut = lds;
-  uint32_t *alut = lds + WLut<BITS>::kDwords;
-  float *partial = reinterpret_cast<float *>(alut + kALutDwords);  // [WAVES][R][64][4]
-
-  fill_lut(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPair, false);
-  fill_lut(alut, g.act_cents, 4, g.a_levels, true, false);
-  __syncthreads();
+  uint32_t *alut = lds + WLut<BITS, kLR>::kDwords;
+  float *partial = reinterpret_cast<float *>(alut + alut_dwords<kLR>());  // [WAVES][R][64][4]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, grp = lane >> 4;
-  const uint32_t wbase = lds_byte_address(wlut) + 4 * (lane & 31);
-  const uint32_t abase = lds_byte_address(alut) + 4 * (lane & 31);
+  const uint32_t wbase = lds_byte_address(wlut) + 4 * (lane & ((1 << kLR) - 1));
+  const uint32_t abase = lds_byte_address(alut) + 4 * (lane & ((1 << kLR) - 1));
   const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * R);
 
   const int steps = static_cast<int>(g.K / 128);
@@ -63,40 +65,103 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     wp[j] = g.w + row * w_row_bytes + grp * (4 * BITS);
   }
 
+  // a batch = kDepth K-steps: every load of the batch is issued before anything waits on it
+  struct Batch {
+    uint4 a[kDepth];
+    uint32_t w[kDepth][R][BITS];
+  };
+  auto fetch = [&](int s0, Batch &bt) {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      const int s = min(s0 + d, s_end - 1);  // clamped: stays inside the row, result unused
+      bt.a[d] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * 64);
+#pragma unroll
+      for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s) * (16 * BITS), bt.w[d][j]);
+    }
+  };
+
   f32x4 acc[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
-  uint4 a_nxt = make_uint4(0, 0, 0, 0);
-  uint32_t w_nxt[R][BITS];
-  if (s_begin < s_end) {
-    a_nxt = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s_begin) * 64);
+  auto consume = [&](int s0, const Batch &bt) {
 #pragma unroll
-    for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s_begin) * (16 * BITS), w_nxt[j]);
-  }
-  for (int s = s_begin; s < s_end; ++s) {
-    const uint4 a_cur = a_nxt;
-    uint32_t w_cur[R][BITS];
+    for (int d = 0; d < kDepth; ++d) {
+      if (s0 + d < s_end) {
 #pragma unroll
-    for (int j = 0; j < R; ++j)
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t f = q == 0 ? bt.a[d].x : q == 1 ? bt.a[d].y : q == 2 ? bt.a[d].z : bt.a[d].w;
+#if defined(OQ_EXP_NOADECODE) || defined(OQ_EXP_NODECODE)
+          const uint4 af = make_uint4(f, f, f, f);
+#else
+          const uint4 af = decode_a_nibble<kLR>(f, abase);
+#endif
 #pragma unroll
-      for (int d = 0; d < BITS; ++d) w_cur[j][d] = w_nxt[j][d];
-    if (s + 1 < s_end) {
-      a_nxt = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s + 1) * 64);
-#pragma unroll
-      for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s + 1) * (16 * BITS), w_nxt[j]);
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t f = q == 0 ? a_cur.x : q == 1 ? a_cur.y : q == 2 ? a_cur.z : a_cur.w;
-      const uint4 af = decode_a_nibble(f, abase);
-#pragma unroll
-      for (int j = 0; j < R; ++j) {
-        const uint4 bf = decode_w<BITS>(w_cur[j], q, wbase);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af), __builtin_bit_cast(bf16x8, bf),
-                                                         acc[j], 0, 0, 0);
+          for (int j = 0; j < R; ++j) {
+#if defined(OQ_EXP_NODECODE)
+            const uint4 bf = make_uint4(bt.w[d][j][0], bt.w[d][j][1 % BITS], bt.w[d][j][BITS - 1], bt.w[d][j][0]);
+#else
+            const uint4 bf = decode_w<BITS, kLR>(bt.w[d][j], q, wbase);
+#endif
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
+                                                             __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
+          }
+        }
       }
     }
+  };
+
+  // Order of the global loads matters: loads of one wavefront return in order, so the few
+  // centroid values the table build needs go first, then both batches of packed data; the
+  // tables are written while the packed data is still in flight.
+  constexpr int kWEntries = WLut<BITS, kLR>::kEntries;
+  const int e_w = tid, e_a = tid - (64 * WAVES - 256);  // last 256 threads build the activation table
+  float wv0 = 0.0f, wv1 = 0.0f, av0 = 0.0f, av1 = 0.0f;
+  if (e_w < kWEntries) {
+    const int c0 = WLut<BITS>::kPair ? (e_w & ((1 << BITS) - 1)) : e_w;
+    const int c1 = WLut<BITS>::kPair ? (e_w >> BITS) : e_w;
+    wv0 = g.w_cents[c0];
+    wv1 = g.w_cents[c1];
+  }
+  if (e_a >= 0) {
+    const int c0 = e_a & 15, c1 = e_a >> 4;
+    av0 = c0 < g.a_levels ? g.act_cents[c0] : 0.0f;
+    av1 = c1 < g.a_levels ? g.act_cents[c1] : 0.0f;
+  }
+  // epilogue operands of the item this thread will finish (item = tid when tid < 64*R)
+  const int ep_j = tid >> 6, ep_l = tid & 63;
+  const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
+  float ep_rn = 0.0f, ep_bv = 0.0f, ep_sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+  if (tid < 64 * R && ep_n < g.N) {
+    ep_rn = bf16_bits_to_f32(g.row_norms[ep_n]);
+    if (g.bias != nullptr) ep_bv = load_dyn_f32(g.bias, g.bias_dtype, ep_n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int m = 4 * (ep_l >> 4) + e;
+      if (g.row_scale != nullptr && m < g.M) ep_sc[e] = g.row_scale[m];
+    }
+  }
+  Batch b0, b1;
+  if (s_begin < s_end) fetch(s_begin, b0);
+  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
+  if (e_w < kWEntries) {
+    const uint32_t d = pack16(wv0, wv1, false);
+    uint4 *dst = reinterpret_cast<uint4 *>(wlut + (e_w << kLR));
+#pragma unroll
+    for (int i = 0; i < (1 << kLR) / 4; ++i) dst[i] = make_uint4(d, d, d, d);
+  }
+  if (e_a >= 0) {
+    const uint32_t d = pack16(av0, av1, false);
+    uint4 *dst = reinterpret_cast<uint4 *>(alut + (e_a << kLR));
+#pragma unroll
+    for (int i = 0; i < (1 << kLR) / 4; ++i) dst[i] = make_uint4(d, d, d, d);
+  }
+  __syncthreads();
+
+  for (int s = s_begin; s < s_end; s += 2 * kDepth) {
+    consume(s, b0);
+    if (s + 2 * kDepth < s_end) fetch(s + 2 * kDepth, b0);
+    if (s + kDepth < s_end) consume(s + kDepth, b1);
+    if (s + 3 * kDepth < s_end) fetch(s + 3 * kDepth, b1);
   }
 
   // ---- cross-wave sum in LDS, fixed order ----------------------------------------
@@ -106,25 +171,19 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
         make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
   __syncthreads();
   // accumulator e of lane l: token row 4*(l/16) + e, weight row l%16
-  for (int item = tid; item < R * 64; item += 64 * WAVES) {
-    const int j = item >> 6, l = item & 63;
-    float4 sum = *reinterpret_cast<const float4 *>(partial + ((0 * R + j) * 64 + l) * 4);
+  if (tid < 64 * R && ep_n < g.N) {
+    float4 sum = *reinterpret_cast<const float4 *>(partial + ((0 * R + ep_j) * 64 + ep_l) * 4);
     for (int w = 1; w < WAVES; ++w) {
-      const float4 p = *reinterpret_cast<const float4 *>(partial + ((w * R + j) * 64 + l) * 4);
+      const float4 p = *reinterpret_cast<const float4 *>(partial + ((w * R + ep_j) * 64 + ep_l) * 4);
       sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
     }
-    const int64_t n = n_base + 16 * j + (l & 15);
-    if (n >= g.N) continue;
-    const float rn = bf16_bits_to_f32(g.row_norms[n]);
-    const float bv = g.bias != nullptr ? load_dyn_f32(g.bias, g.bias_dtype, n) : 0.0f;
     const float v[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int m = 4 * (l >> 4) + e;
+      const int m = 4 * (ep_l >> 4) + e;
       if (m >= g.M) continue;
-      const float sc = g.row_scale != nullptr ? g.row_scale[m] : 1.0f;
-      const float y = v[e] * sc * rn + bv;
-      const int64_t o = static_cast<int64_t>(m) * g.N + n;
+      const float y = v[e] * ep_sc[e] * ep_rn + ep_bv;
+      const int64_t o = static_cast<int64_t>(m) * g.N + ep_n;
       if (g.out_dtype == OQ_BF16) static_cast<uint16_t *>(g.out)[o] = f32_to_bf16_bits(y);
       else if (g.out_dtype == OQ_F16) static_cast<uint16_t *>(g.out)[o] = f32_to_f16_bits(y);
       else static_cast<float *>(g.out)[o] = y;
@@ -136,7 +195,7 @@ template <int BITS, int R, int WAVES>
 int launch(const GemvArgs &g, hipStream_t stream) {
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
   if (groups > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: N too large");
-  const size_t smem = (WLut<BITS>::kDwords + kALutDwords) * sizeof(uint32_t) + sizeof(float) * WAVES * R * 64 * 4;
+  const size_t smem = (WLut<BITS, kLR>::kDwords + alut_dwords<kLR>()) * sizeof(uint32_t) + sizeof(float) * WAVES * R * 64 * 4;
   auto kern = packed_gemv_kernel<BITS, R, WAVES>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -147,11 +206,27 @@ int launch(const GemvArgs &g, hipStream_t stream) {
   return check_launch("packed_gemv");
 }
 
+template <int BITS, int R>
+int launch_waves(const GemvArgs &g, int waves, hipStream_t stream) {
+  if (waves == 4) return launch<BITS, R, 4>(g, stream);
+  if (waves == 16) return launch<BITS, R, 16>(g, stream);
+  return launch<BITS, R, 8>(g, stream);
+}
+
 template <int BITS>
 int launch_bits(const GemvArgs &g, hipStream_t stream) {
-  // 16 rows per workgroup while that still leaves fewer than ~2 workgroups per CU, else 32
-  if (g.N <= 16 * 512) return launch<BITS, 1, 8>(g, stream);
-  return launch<BITS, 2, 8>(g, stream);
+  // rows per workgroup (16*R) and K-split (wavefronts per workgroup); OQ_GEMV_CFG="R,WAVES" overrides
+  int r = g.N <= 16 * 512 ? 1 : 2, waves = 8;
+  if (const char *cfg = getenv("OQ_GEMV_CFG")) {
+    int cr = 0, cw = 0;
+    if (sscanf(cfg, "%d,%d", &cr, &cw) == 2 && (cr == 1 || cr == 2 || cr == 4) && (cw == 4 || cw == 8 || cw == 16)) {
+      r = cr;
+      waves = cw;
+    }
+  }
+  if (r == 1) return launch_waves<BITS, 1>(g, waves, stream);
+  if (r == 4) return launch_waves<BITS, 4>(g, waves, stream);
+  return launch_waves<BITS, 2>(g, waves, stream);
 }
 
 }  // namespace
