@@ -90,6 +90,9 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int64_t m_base = static_cast<int64_t>(pid_m) * TM + (wave >> 1) * (FM * 32);
   const int64_t n_base = static_cast<int64_t>(pid_n) * TN + (wave & 1) * (FN * 32);
 
+  EpiFactors<FM> epi;
+  gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, (wave >> 1) * (FM * 32), TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+
   constexpr int A_ROW_STEP = AM == A_NIBBLE ? 32 : 128;  // bytes of one row consumed per K-step of 64
   constexpr int A_GRP_OFF = AM == A_NIBBLE ? 16 : 64;
   const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K * 2;
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(af[i], bf[j], acc[i][j]);
+      for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(bf[j], af[i], acc[i][j]);  // weights first: transposed tile
   };
   // interleave hint: after each MFMA, the lookups' address arithmetic and LDS reads
   constexpr int kLookupsPerMfma = (AM == A_NIBBLE ? (FM + FN) : FN) * 4 / (FM * FN);
@@ -197,8 +200,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     interleave();
   }
 
-  gemm_epilogue<FM, FN>(acc, m_base, n_base, r, grp, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.out,
-                        g.out_dtype);
+  __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused by the epilogue
+  gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, (wave >> 1) * (FM * 32),
+                        (wave & 1) * (FN * 32), TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
+                        g.out_dtype, reinterpret_cast<unsigned char *>(lds));
 }
 
 template <int AM, int BITS, int FM, int FN>
@@ -208,7 +213,8 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  const size_t smem = (WLut<BITS>::kDwords + (AM == A_NIBBLE ? kALutDwords : 0)) * sizeof(uint32_t);
+  size_t smem = (WLut<BITS>::kDwords + (AM == A_NIBBLE ? kALutDwords : 0)) * sizeof(uint32_t);
+  if (smem < static_cast<size_t>(kEpiLdsBytes)) smem = kEpiLdsBytes;  // the epilogue reuses LDS
   auto kern = packed_gemm_kernel<AM, BITS, FM, FN>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -78,6 +78,9 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
   const int64_t m0 = static_cast<int64_t>(pid_m) * TM, n0 = static_cast<int64_t>(pid_n) * TN;
   const int wm = (wave >> 1) * (FM * 32), wn = (wave & 1) * (FN * 32);
 
+  EpiFactors<FM> epi;
+  gemm_epilogue_prefetch<FM>(epi, m0, n0, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+
   // ---- A loader: chunk c = tid + 256*i -> row c/8, 16-byte chunk c%8 of the row's 128-byte slab
   const int64_t a_row_bytes = g.K * 2, w_row_bytes = g.K * BITS / 8;
   const int ld_row = tid >> 3, ld_off = (tid & 7) * 16;
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j) acc[i][j] = mfma16<F16>(af[i], bf[j], acc[i][j]);
+      for (int j = 0; j < FN; ++j) acc[i][j] = mfma16<F16>(bf[j], af[i], acc[i][j]);  // weights first: transposed tile
   };
 
   // ---- prologue: slabs 0 and 1 into LDS, slab 2 and the weights of K-step 1 in flight ----
@@ -176,8 +179,9 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
     multiply(af1, bf1);
   }
 
-  gemm_epilogue<FM, FN>(acc, m0 + wm, n0 + wn, r, grp, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.out,
-                        g.out_dtype);
+  __syncthreads();  // tables and staging buffers are dead: LDS is reused by the epilogue
+  gemm_epilogue<FM, FN>(acc, m0, n0, wm, wn, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
+                        g.out_dtype, reinterpret_cast<unsigned char *>(lds));
 }
 
 template <bool F16, int BITS, int FM, int FN>
@@ -187,7 +191,8 @@ int launch_cfg(AvArgs g, hipStream_t stream) {
   g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  const size_t smem = WLut<BITS>::kDwords * sizeof(uint32_t) + 2 * static_cast<size_t>(TM) * kAPitch;
+  size_t smem = WLut<BITS>::kDwords * sizeof(uint32_t) + 2 * static_cast<size_t>(TM) * kAPitch;
+  if (smem < static_cast<size_t>(kEpiLdsBytes)) smem = kEpiLdsBytes;  // the epilogue reuses LDS
   auto kern = packed_gemm_av_kernel<F16, BITS, FM, FN>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -100,6 +100,9 @@ __global__ __launch_bounds__(256) void packed_gemm_staged_kernel(StagedArgs g) {
   const int64_t m0 = static_cast<int64_t>(pid_m) * TM, n0 = static_cast<int64_t>(pid_n) * TN;
   const int wm = (wave >> 1) * (FM * 32), wn = (wave & 1) * (FN * 32);
 
+  EpiFactors<FM> epi;
+  gemm_epilogue_prefetch<FM>(epi, m0, n0, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+
   // ---- loader assignment: chunk c = tid + 256*i -> (row c / CH, 16-byte chunk c % CH) ----
   const int64_t a_row_bytes = g.K / 2, w_row_bytes = g.K * BITS / 8;
   const uint8_t *a_src[A_PER_T];
@@ -176,8 +179,8 @@ __global__ __launch_bounds__(256) void packed_gemm_staged_kernel(StagedArgs g) {
         for (int i = 0; i < FM; ++i)
 #pragma unroll
           for (int j = 0; j < FN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i]),
-                                                                __builtin_bit_cast(bf16x8, bf[j]), acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bf[j]),
+                                                                __builtin_bit_cast(bf16x8, af[i]), acc[i][j], 0, 0, 0);
       }
     }
     if (s + 1 < slabs) {
@@ -186,8 +189,9 @@ __global__ __launch_bounds__(256) void packed_gemm_staged_kernel(StagedArgs g) {
     }
   }
 
-  gemm_epilogue<FM, FN>(acc, m0 + wm, n0 + wn, r, grp, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.out,
-                        g.out_dtype);
+  __syncthreads();  // tables and staging buffers are dead: LDS is reused by the epilogue
+  gemm_epilogue<FM, FN>(acc, m0, n0, wm, wn, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
+                        g.out_dtype, reinterpret_cast<unsigned char *>(lds));
 }
 
 template <int BITS, int FM, int FN, int KS>
@@ -197,8 +201,9 @@ int launch_cfg(StagedArgs g, hipStream_t stream) {
   g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  const size_t smem = (WLut<BITS>::kDwords + kALutDwords) * sizeof(uint32_t) +
+  size_t smem = (WLut<BITS>::kDwords + kALutDwords) * sizeof(uint32_t) +
                       2 * (static_cast<size_t>(TM) * odd16(KS / 2) + static_cast<size_t>(TN) * odd16(KS * BITS / 8));
+  if (smem < static_cast<size_t>(kEpiLdsBytes)) smem = kEpiLdsBytes;  // the epilogue reuses LDS
   auto kern = packed_gemm_staged_kernel<BITS, FM, FN, KS>;
   if (smem > 160 * 1024) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: tile needs %zu bytes of LDS", smem);
   if (smem > 48 * 1024) {
