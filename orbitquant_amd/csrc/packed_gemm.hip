@@ -65,9 +65,23 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   uint32_t *wlut = lds;
   uint32_t *alut = lds + WLut<BITS>::kDwords;
 
-  fill_lut(wlut, g.w_cents, BITS, 1 << BITS, WLut<BITS>::kPair, AM == A_F16);
-  if constexpr (AM == A_NIBBLE) fill_lut(alut, g.act_cents, 4, g.a_levels, true, false);
-  __syncthreads();
+  // Loads of one wavefront return in order, so the handful of centroid values this thread
+  // needs for its table entries are requested first, then the packed operands of the first
+  // two K-steps; the tables are written while the packed data is still in flight.
+  constexpr int kWEntries = WLut<BITS>::kEntries;
+  float lut_w0 = 0.0f, lut_w1 = 0.0f, lut_a0 = 0.0f, lut_a1 = 0.0f;
+  {
+    const int e = threadIdx.x;
+    if (e < kWEntries) {
+      lut_w0 = g.w_cents[WLut<BITS>::kPair ? (e & ((1 << BITS) - 1)) : e];
+      lut_w1 = g.w_cents[WLut<BITS>::kPair ? (e >> BITS) : e];
+    }
+    if constexpr (AM == A_NIBBLE) {
+      const int c0 = e & 15, c1 = e >> 4;
+      lut_a0 = c0 < g.a_levels ? g.act_cents[c0] : 0.0f;
+      lut_a1 = c1 < g.a_levels ? g.act_cents[c1] : 0.0f;
+    }
+  }
 
   constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
   // tile order: spread consecutive workgroup ids over the 8 XCDs' private L2s in
@@ -137,6 +151,23 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + 8 * BITS, w_nxt[j]);
   }
+
+  {  // table entries: one per thread, 32 copies each
+    const int e = threadIdx.x;
+    if (e < kWEntries) {
+      const uint32_t d = pack16(lut_w0, lut_w1, AM == A_F16);
+      uint4 *dst = reinterpret_cast<uint4 *>(wlut + e * 32);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i] = make_uint4(d, d, d, d);
+    }
+    if constexpr (AM == A_NIBBLE) {
+      const uint32_t d = pack16(lut_a0, lut_a1, false);
+      uint4 *dst = reinterpret_cast<uint4 *>(alut + e * 32);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i] = make_uint4(d, d, d, d);
+    }
+  }
+  __syncthreads();
 
   auto decode = [&](int q, uint4 (&af)[FM], uint4 (&bf)[FN]) {
 #pragma unroll
