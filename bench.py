@@ -189,39 +189,101 @@ def quantize_only_closure(layer, x):
 
 # ----------------------------------------------------------------- CPU baseline
 
-def cpu_baseline(spec, layers, x, budget_rows):
-    """Oracle (CPU port of the reference path) on the first `budget_rows` tokens: per layer
-    rotate+quantize to values, then the scalar packed matmul with fp32 accumulation."""
-    from oracle import oracle_c, oracle_np
+def _cpu_threads() -> int:
+    """Thread count of the CPU leg: what the box grants (OMP_NUM_THREADS when set, else the
+    affinity mask), capped at 64 like the reference's pool (cpu_threads.cpp:22-36,89-101)."""
+    env = os.environ.get("ORBITQUANT_CPU_THREADS") or os.environ.get("OMP_NUM_THREADS")
+    n = int(env) if env and env.isdigit() and int(env) > 0 else len(os.sched_getaffinity(0))
+    return max(1, min(n, 64))
 
-    threads = oracle_c.max_threads()
-    rows = min(budget_rows, x.shape[0])
-    h = x[:rows].float().cpu().numpy()
-    flops = 0.0
+
+def cpu_baseline(spec, layers, x, target_seconds=15.0):
+    """The CPU path on a bounded sample of the same workload, about `target_seconds` of work.
+
+    kind "reference": the reference's own CPU kernels (quantize_activations_cpu +
+    matmul_packed_weight, compiled from the reference checkout into oracle/_ref) when that
+    library travelled with the tree; else kind "port": the C oracle.  Same layers, same
+    packed weights, same activations as the GPU leg."""
+    from oracle import oracle_c, ref_cpu
+
+    threads = _cpu_threads()
+    os.environ["ORBITQUANT_CPU_THREADS"] = str(threads)   # read by the reference's pool on first use
+    use_ref = ref_cpu.available()
     prepared = []
     for layer, act in layers:
         prepared.append(dict(
-            perm=layer.rotation.permutation.numpy().astype(np.int32), signs=layer.rotation.signs.numpy(),
-            bounds=layer.activation_codebook.boundaries.numpy(), cents=layer.activation_codebook.centroids.numpy(),
-            block=layer.rotation.block_size, inv=np.float32(layer.rotation.normalization),
-            packed=layer.packed_weight_indices.cpu().numpy(), r=layer.row_norms.float().cpu().numpy(),
-            cw=layer.weight_codebook.centroids.numpy(), bits=layer.weight_bits, n=layer.out_features,
-            k=layer.in_features, act=act))
+            perm=layer.rotation.permutation.to(torch.int32), signs=layer.rotation.signs.to(torch.int8),
+            bounds=layer.activation_codebook.boundaries.float(), cents=layer.activation_codebook.centroids.float(),
+            block=layer.rotation.block_size, inv=float(np.float32(layer.rotation.normalization)),
+            packed=layer.packed_weight_indices.cpu(), r=layer.row_norms.float().cpu(),
+            cw=layer.weight_codebook.centroids.float(), bits=layer.weight_bits, n=layer.out_features,
+            k=layer.in_features, act=act, bias=None if layer.bias is None else layer.bias.float().cpu()))
+
+    def run(rows):
+        h = x[:rows].cpu()
+        for p in prepared:
+            if use_ref:
+                q = ref_cpu.quantize_activations_cpu(h, p["perm"], p["signs"], p["cents"], p["bounds"], eps=1e-10,
+                                                     inv_sqrt_block=p["inv"], block_size=p["block"])
+                y = ref_cpu.matmul_packed_weight(q, p["packed"], p["r"], p["cw"], bits=p["bits"],
+                                                 out_features=p["n"], in_features=p["k"], bias=p["bias"])
+            else:
+                codes, s = oracle_c.rotate_quantize(h.float().numpy(), p["perm"].numpy(), p["signs"].numpy(),
+                                                    p["bounds"].numpy(), p["block"], 1e-10, np.float32(p["inv"]),
+                                                    threads)
+                vals = p["cents"].numpy()[codes] * s[:, None]
+                y = torch.from_numpy(oracle_c.matmul_packed_weight(
+                    vals, p["packed"].numpy(), p["r"].numpy(), p["cw"].numpy(),
+                    None if p["bias"] is None else p["bias"].numpy(), p["bits"], p["n"], threads)).to(h.dtype)
+            if p["act"] == "gelu":
+                y = torch.nn.functional.gelu(y)
+            elif p["act"] == "slice3072":
+                y = y[:, :3072].contiguous()
+            h = y
+
+    m = x.shape[0]
+    rows0 = min(m, 64)
+    run(rows0)                                   # warm-up: thread pool, page-in
     t0 = time.perf_counter()
-    for p in prepared:
-        codes, s = oracle_c.rotate_quantize(h, p["perm"], p["signs"], p["bounds"], p["block"], 1e-10, p["inv"], threads)
-        vals = p["cents"][codes] * s[:, None]
-        y = oracle_c.matmul_packed_weight(vals, p["packed"], p["r"], p["cw"], None, p["bits"], p["n"], threads)
-        flops += 2.0 * rows * p["n"] * p["k"]
-        if p["act"] == "gelu":
-            y = torch.nn.functional.gelu(torch.from_numpy(y)).numpy()
-        elif p["act"] == "slice3072":
-            y = np.ascontiguousarray(y[:, :3072])
-        h = y
+    run(rows0)
+    per_row = (time.perf_counter() - t0) / rows0
+    rows = int(min(m, max(rows0, target_seconds / per_row)))
+    reps = max(1, int(round(target_seconds / (per_row * rows)))) if rows == m else 1
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run(rows)
     dt = time.perf_counter() - t0
-    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=threads, kind="port",
-                sample=f"first {rows} of {x.shape[0]} tokens through every layer of the workload, {dt:.2f} s, "
-                       f"oracle/oq_oracle.c with OpenMP ({os.cpu_count()} logical CPUs visible)")
+    flops = reps * sum(2.0 * rows * p["n"] * p["k"] for p in prepared)
+    what = ("reference CPU kernels (quantize_activations_cpu + matmul_packed_weight) built into oracle/_ref"
+            if use_ref else "oracle/oq_oracle.c with OpenMP")
+    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=threads, kind="reference" if use_ref else "port",
+                sample=f"{reps} pass(es) over the first {rows} of {m} tokens through every layer of the workload, "
+                       f"{dt:.1f} s, {what}, {threads} threads")
+
+
+def copy_calibration(device, launches=3, mib=256):
+    """A plain device copy of known size (`mib` MiB read + `mib` MiB written per launch), so that a
+    profiler run of this script holds the yardstick its FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    src = torch.empty(mib << 20, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(launches):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
+def recorded_traffic(key: str):
+    """HBM bytes per launch of the dominant kernel, measured with the profiler's FETCH_SIZE and WRITE_SIZE
+    counters and written down in profiles/ (a live run cannot read those counters itself)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.txt")
+    try:
+        with open(path) as fh:
+            for line in fh:
+                parts = line.split()
+                if len(parts) >= 2 and parts[0] == key:
+                    return float(parts[1])
+    except OSError:
+        pass
+    return None
 
 
 # ------------------------------------------------------------------------ c5
@@ -304,11 +366,12 @@ def bench_c5(args, device):
         "data": "synthetic", "config": {"workload": f"c5 40-layer decode stack W2/W3/W4 A4, M={m}", "M": m,
                                         "packed_bytes_per_step": packed_bytes},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("c5_gemv_w4_4096x14336"),
                      "kernel": "packed_gemv_kernel<4> on 4096->14336 W4", "bytes_per_launch": w4_bytes,
                      "avg_launch_us": per_w4 * 1e6,
                      "stack_matmuls_gbs": packed_bytes / per_stack / 1e9},
     }
+    copy_calibration(device)
     print(json.dumps(out))
 
 
@@ -369,13 +432,13 @@ def main() -> int:
         "config": {"workload": spec["name"], "M": spec["M"], "input_dtype": str(spec["dtype"]).replace("torch.", ""),
                    "flop_per_step": flops},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded_traffic(f"{args.workload}_gemm"),
                      "kernel": "packed_gemm_kernel", "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},
         "pieces": pieces,
     }
+    copy_calibration(device)
     if not args.no_cpu_baseline:
-        budget = {"c1": 256, "c2": 256, "c3": 48, "c4": 32}[args.workload]
-        out["cpu_baseline"] = cpu_baseline(spec, layers, x, budget)
+        out["cpu_baseline"] = cpu_baseline(spec, layers, x)
     print(json.dumps(out))
     return 0
 

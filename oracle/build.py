@@ -29,30 +29,30 @@ def build_oracle() -> Path:
 
 
 def build_reference_cpu() -> Path | None:
-    """Compile the reference's scalar/AVX2/AVX-512 packed-matmul range kernels
-    from where they lie, plus this repo's C-ABI shim around their C++ interface.
-    Returns None when the reference checkout (or torch's header-only BFloat16/
-    Half headers it includes) is not present."""
-    shim = HERE / "ref_cpu_shim.cpp"
-    if not REF_CPU.is_dir() or not shim.exists():
+    """Compile the reference's CPU kernels on this path (packed matmul + activation
+    quantizer, with their thread pool and ISA dispatch) from where they lie, plus this
+    repo's own operator registration (`ref_cpu_bind.cpp`), into oracle/_ref/.  The
+    reference's generated binding glue is not used.  Returns None when the reference
+    checkout is not present (e.g. on a GPU box, which only uses a prebuilt file)."""
+    bind = HERE / "ref_cpu_bind.cpp"
+    if not REF_CPU.is_dir():
         return None
-    try:
-        import torch
-    except Exception:
-        return None
-    include = Path(torch.__file__).resolve().parent / "include"
-    if not (include / "torch/headeronly/util/BFloat16.h").exists():
-        return None
+    from torch.utils import cpp_extension
+
+    import torch
+
     REF_DIR.mkdir(exist_ok=True)
-    sources = [
-        REF_CPU / "packed_matmul_scalar.cpp",
-        REF_CPU / "packed_matmul_x86.cpp",
-        REF_CPU / "packed_matmul_x86_avx512.cpp",
-    ]
+    names = ["packed_matmul_cpu", "packed_matmul_scalar", "packed_matmul_x86", "packed_matmul_x86_avx512",
+             "packed_matmul_neon", "quantize_activations_cpu", "cpu_pool", "cpu_threads", "cpu_isa"]
+    sources = [REF_CPU / f"{n}.cpp" for n in names]
+    includes = [f"-I{p}" for p in cpp_extension.include_paths()]
+    lib_dir = Path(torch.__file__).resolve().parent / "lib"
     cmd = [
-        "g++", "-std=c++17", "-O3", "-fopenmp", "-shared", "-fPIC",
-        f"-I{REF_CPU}", f"-I{include}", "-o", str(REF_SO), str(shim),
-    ] + [str(s) for s in sources]
+        "g++", "-std=c++17", "-O3", "-DCPU_KERNEL", "-shared", "-fPIC", "-pthread",
+        f"-I{REF_CPU}", f"-I{REF_CPU.parent / 'torch-ext'}", *includes,
+        "-o", str(REF_SO), str(bind), *[str(s) for s in sources],
+        f"-L{lib_dir}", "-ltorch", "-ltorch_cpu", "-lc10", f"-Wl,-rpath,{lib_dir}",
+    ]
     subprocess.run(cmd, check=True)
     return REF_SO
 
