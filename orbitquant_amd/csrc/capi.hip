@@ -4,7 +4,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#include "oq_common.h"
+#include "gemm_epilogue.h"
 
 namespace oq {
 
@@ -125,13 +125,14 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
   const int a_levels = 1 << a_bits;
   hipStream_t s = as_stream(stream);
   const bool fast_ptrs = aligned16(codes) && aligned16(packed_w);
+  const bool tiled_out = gemm_output_ok(N, out);  // the tiled kernels store 16-byte row segments
   if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
     return gemv_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
-  if (fast_ptrs && code_format == OQ_CODES_NIBBLE && gemm_staged_supported(K, w_bits) && getenv("OQ_GEMM_STAGED") != nullptr)
+  if (fast_ptrs && tiled_out && code_format == OQ_CODES_NIBBLE && gemm_staged_supported(K, w_bits) && getenv("OQ_GEMM_STAGED") != nullptr)
     return gemm_staged_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                                 bias, bias_dtype, M, N, K, out, out_dtype, gemm_choose_tile(M, N), s);
-  if (fast_ptrs && code_format == OQ_CODES_NIBBLE && gemm_supported(K, w_bits))
+  if (fast_ptrs && tiled_out && code_format == OQ_CODES_NIBBLE && gemm_supported(K, w_bits))
     return gemm_dispatch(0, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
   return generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
@@ -146,7 +147,7 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   if (M == 0) return OQ_OK;
   if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
   hipStream_t s = as_stream(stream);
-  if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_av_supported(K, bits))
+  if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
     return gemm_av_dispatch(x_dtype == OQ_F16, x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype,
                             M, N, K, out, out_dtype, gemm_choose_tile(M, N), s);
   return generic_matmul_float(x, x_dtype, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N,

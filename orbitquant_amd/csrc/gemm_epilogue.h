@@ -4,22 +4,38 @@
 // an accumulator tile is the transpose of the output tile: value e of lane l is
 //   token row   m = 32*i + l%32
 //   output col  n = 32*j + 8*(e/4) + 4*(l/32) + e%4
-// i.e. every lane holds runs of four consecutive columns of one output row.  The
-// fast path scales a run, packs it (8 bytes of bf16/fp16, 16 of fp32) and parks it
-// in a wavefront-private LDS tile; the tile is then read back row-wise, 16 bytes
-// per lane, so the global stores are whole 128-byte (or longer) row segments
-// instead of 2-byte scatters.  Per-column factors (row norm, bias) are staged in
-// LDS once per workgroup.
+// i.e. every lane holds runs of four consecutive columns of one output row.
+//
+// A wavefront moves its tiles to memory in passes of [32 rows x 64 columns]
+// through a private fp32 staging tile in LDS:
+//   1. every lane writes its raw accumulator runs (16 bytes per ds_write, straight
+//      from the accumulator registers) - no arithmetic, no reads, nothing to wait for;
+//   2. the tile is read back row-wise, each lane taking eight consecutive columns
+//      of one row; it multiplies by the token factor of that row (staged in LDS)
+//      and the row norms and adds the bias (both held in registers for the whole
+//      column block), converts and stores 16 bytes (bf16 / fp16; 2 x 16 for fp32),
+//      so a store instruction writes whole 128-byte row segments.
+// LDS operations of one wavefront execute in program order, so step 2 of a pass
+// needs no barrier after step 1, and step 1 of the next pass may be issued as soon
+// as the reads of step 2 have been issued.  The cost is instruction issue: about
+// 2.5 vector instructions per output value.
+//
+// Needs N % 8 == 0 and a 16-byte aligned `out` (the dispatcher sends other
+// shapes to the shape-agnostic kernels).
 #pragma once
 
 #include "packed_decode.h"
 
 namespace oq {
 
-constexpr int kEpiFactorBytes = 2048;                 // r_w[256] + bias[256] as fp32
-constexpr int kEpiWavePitchMax = 32 * 2 * 4 + 16;     // two 32-column tiles of fp32 + padding
-constexpr int kEpiWaveBytes = 32 * kEpiWavePitchMax;  // 8704
+constexpr int kEpiFactorBytes = 3072;            // r_w[256] + bias[256] + token factor[256] as fp32
+constexpr int kEpiPitch = 64 * 4 + 16;           // one staged row: 64 fp32 + padding
+constexpr int kEpiWaveBytes = 32 * kEpiPitch;    // 8704
 constexpr int kEpiLdsBytes = kEpiFactorBytes + 4 * kEpiWaveBytes;
+
+inline bool gemm_output_ok(int64_t N, const void *out) {
+  return (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
+}
 
 // Per-thread epilogue factors, loaded at kernel start so their latency hides behind the main loop:
 // thread t < tile_n owns output column n_tile + t; every lane owns the token rows wm + 32*i + lane%32.
@@ -46,100 +62,91 @@ __device__ __forceinline__ void gemm_epilogue_prefetch(EpiFactors<FM> &f, int64_
     f.sc[i] = row_scale != nullptr ? row_scale[min(m_tile + wm + 32 * i + (tid & 31), M - 1)] : 1.0f;
 }
 
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// two fp32 -> one dword of two 16-bit floats (round to nearest even), one conversion instruction
 template <int OUT_DT>
-__device__ __forceinline__ void pack_run(const float (&y)[4], unsigned char *dst) {
-  if constexpr (OUT_DT == OQ_F32) {
-    *reinterpret_cast<float4 *>(dst) = make_float4(y[0], y[1], y[2], y[3]);
-  } else if constexpr (OUT_DT == OQ_BF16) {
-    uint2 v;
-    v.x = static_cast<uint32_t>(f32_to_bf16_bits(y[0])) | (static_cast<uint32_t>(f32_to_bf16_bits(y[1])) << 16);
-    v.y = static_cast<uint32_t>(f32_to_bf16_bits(y[2])) | (static_cast<uint32_t>(f32_to_bf16_bits(y[3])) << 16);
-    *reinterpret_cast<uint2 *>(dst) = v;
-  } else {
-    uint2 v;
-    v.x = static_cast<uint32_t>(f32_to_f16_bits(y[0])) | (static_cast<uint32_t>(f32_to_f16_bits(y[1])) << 16);
-    v.y = static_cast<uint32_t>(f32_to_f16_bits(y[2])) | (static_cast<uint32_t>(f32_to_f16_bits(y[3])) << 16);
-    *reinterpret_cast<uint2 *>(dst) = v;
-  }
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  if constexpr (OUT_DT == OQ_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
 }
 
-// Fast path.  `lds` = start of kEpiLdsBytes of LDS nobody else uses any more (the caller
-// has put a barrier between the main loop and this call).  Needs N % 8 == 0 and a
-// 16-byte aligned `out`.
-template <int FM, int FN, int OUT_DT>
-__device__ __forceinline__ void gemm_epilogue_lds(const f32x16 (&acc)[FM][FN], int64_t m_tile, int64_t n_tile,
-                                                  int wm, int wn, int tile_n, int tid, int64_t M, int64_t N,
-                                                  const EpiFactors<FM> &pre, void *__restrict__ out,
-                                                  unsigned char *lds) {
-  constexpr int ES = OUT_DT == OQ_F32 ? 4 : 2;
-  constexpr int JC = FN >= 2 ? 2 : 1;             // 32-column tiles per pass
-  constexpr int ROW_BYTES = 32 * JC * ES;
-  constexpr int PITCH = ROW_BYTES + 16;
-  constexpr int LPR = ROW_BYTES / 16;             // lanes per row when reading back
-  constexpr int RPI = 64 / LPR;                   // rows per read instruction
+// `lds` = start of kEpiLdsBytes of LDS nobody else uses any more (the caller has put a
+// barrier between its main loop and this call).
+// GUARD = false: the workgroup's tile lies wholly inside the output, no store is predicated
+// (one straight-line block, so LDS reads, arithmetic and stores of different rows overlap).
+template <int FM, int FN, int OUT_DT, bool GUARD>
+__device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN], int64_t m_tile, int64_t n_tile,
+                                                    int wm, int wn, int tile_n, int tid, int64_t M, int64_t N,
+                                                    const EpiFactors<FM> &pre, void *__restrict__ out,
+                                                    unsigned char *lds) {
   const int lane = tid & 63, wave = tid >> 6, r = lane & 31, grp = lane >> 5;
 
+  constexpr int ES = OUT_DT == OQ_F32 ? 4 : 2;
   float *rn_s = reinterpret_cast<float *>(lds);
   float *bv_s = rn_s + 256;
+  float *sc_s = rn_s + 512;
   if (tid < tile_n) {
     rn_s[tid] = pre.rn;
     bv_s[tid] = pre.bv;
   }
+  if (wn == 0 && grp == 0) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) sc_s[wm + 32 * i + r] = pre.sc[i];
+  }
   __syncthreads();
   unsigned char *tile = lds + kEpiFactorBytes + wave * kEpiWaveBytes;
+  const int64_t row_pitch = N * ES;  // bytes between output rows
 
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const float sc = pre.sc[i];
+  for (int jc = 0; jc < FN; jc += 2) {
+    constexpr int kTwo = 2;
+    const int JC = (FN - jc) < kTwo ? 1 : 2;     // 32-column tiles in this pass (compile-time after unrolling)
+    const int LPR = 4 * JC;                      // lanes per row when reading back (8 columns each)
+    const int RPI = 64 / LPR;                    // rows per read instruction
+    const int row0 = lane / LPR, c = lane % LPR;
+    // this lane's eight columns of the block: factors stay in registers for every row tile
+    const float4 rn0 = *reinterpret_cast<const float4 *>(rn_s + wn + 32 * jc + 8 * c);
+    const float4 rn1 = *reinterpret_cast<const float4 *>(rn_s + wn + 32 * jc + 8 * c + 4);
+    const float4 bv0 = *reinterpret_cast<const float4 *>(bv_s + wn + 32 * jc + 8 * c);
+    const float4 bv1 = *reinterpret_cast<const float4 *>(bv_s + wn + 32 * jc + 8 * c + 4);
+    const int64_t nn = n_tile + wn + 32 * jc + 8 * c;
+    const int64_t m_first = m_tile + wm + row0;
+    unsigned char *dst = static_cast<unsigned char *>(out) + m_first * row_pitch + nn * ES;
+    const int rows_left = static_cast<int>(min(static_cast<int64_t>(FM * 32), M - m_first));  // rows m_first+k, k < rows_left, exist
+    const bool col_ok = nn < N;
 #pragma unroll
-    for (int jc = 0; jc < FN; jc += JC) {
+    for (int i = 0; i < FM; ++i) {
 #pragma unroll
-      for (int jj = 0; jj < JC; ++jj) {
+      for (int jj = 0; jj < JC; ++jj)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-          const int col = 32 * jj + 8 * a + 4 * grp;  // inside this pass
-          const float4 rn = *reinterpret_cast<const float4 *>(rn_s + wn + 32 * jc + col);
-          const float4 bv = *reinterpret_cast<const float4 *>(bv_s + wn + 32 * jc + col);
-          const float y[4] = {acc[i][jc + jj][4 * a + 0] * sc * rn.x + bv.x, acc[i][jc + jj][4 * a + 1] * sc * rn.y + bv.y,
-                              acc[i][jc + jj][4 * a + 2] * sc * rn.z + bv.z, acc[i][jc + jj][4 * a + 3] * sc * rn.w + bv.w};
-          pack_run<OUT_DT>(y, tile + r * PITCH + col * ES);
+          const int col = 32 * jj + 8 * a + 4 * grp;
+          *reinterpret_cast<float4 *>(tile + r * kEpiPitch + col * 4) =
+              make_float4(acc[i][jc + jj][4 * a + 0], acc[i][jc + jj][4 * a + 1], acc[i][jc + jj][4 * a + 2],
+                          acc[i][jc + jj][4 * a + 3]);
         }
-      }
-      // read the [32 x 32*JC] tile back row-wise and store whole row segments
 #pragma unroll
       for (int t = 0; t < 32 / RPI; ++t) {
-        const int row = t * RPI + lane / LPR, c = lane % LPR;
-        const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * PITCH + c * 16);
-        const int64_t mm = m_tile + wm + 32 * i + row;
-        const int64_t nn = n_tile + wn + 32 * jc + c * (16 / ES);
-        if (mm < M && nn < N)
-          *reinterpret_cast<uint4 *>(static_cast<unsigned char *>(out) + (mm * N + nn) * ES) = v;
-      }
-    }
-  }
-}
-
-// Fallback for unaligned outputs / N not a multiple of 8: one store per value.
-template <int FM, int FN, int OUT_DT>
-__device__ __forceinline__ void gemm_epilogue_scalar(const f32x16 (&acc)[FM][FN], int64_t m_base, int64_t n_base,
-                                                     int r, int grp, int64_t M, int64_t N,
-                                                     const float *__restrict__ row_scale,
-                                                     const uint16_t *__restrict__ row_norms,
-                                                     const void *__restrict__ bias, int bias_dtype,
-                                                     void *__restrict__ out) {
-#pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int64_t m = m_base + 32 * i + r;
-    const float sc = row_scale != nullptr ? row_scale[min(m, M - 1)] : 1.0f;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll 1
-      for (int e = 0; e < 16; ++e) {
-        const int64_t n = n_base + 32 * j + 8 * (e >> 2) + 4 * grp + (e & 3);
-        if (m < M && n < N) {
-          const float rn = bf16_bits_to_f32(row_norms[n]);
-          const float bv = bias != nullptr ? load_dyn_f32(bias, bias_dtype, n) : 0.0f;
-          store_from_f32<OUT_DT>(out, m * N + n, acc[i][j][e] * sc * rn + bv);
+        const int row = t * RPI + row0;
+        const float4 v0 = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32);
+        const float4 v1 = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32 + 16);
+        const float sc = sc_s[wm + 32 * i + row];
+        const float y[8] = {(v0.x * sc) * rn0.x + bv0.x, (v0.y * sc) * rn0.y + bv0.y, (v0.z * sc) * rn0.z + bv0.z,
+                            (v0.w * sc) * rn0.w + bv0.w, (v1.x * sc) * rn1.x + bv1.x, (v1.y * sc) * rn1.y + bv1.y,
+                            (v1.z * sc) * rn1.z + bv1.z, (v1.w * sc) * rn1.w + bv1.w};
+        if (!GUARD || (col_ok && 32 * i + t * RPI < rows_left)) {
+          unsigned char *o = dst + (32 * i + t * RPI) * row_pitch;
+          if constexpr (OUT_DT == OQ_F32) {
+            reinterpret_cast<float4 *>(o)[0] = make_float4(y[0], y[1], y[2], y[3]);
+            reinterpret_cast<float4 *>(o)[1] = make_float4(y[4], y[5], y[6], y[7]);
+          } else {
+            *reinterpret_cast<uint4 *>(o) = make_uint4(pack_pair<OUT_DT>(y[0], y[1]), pack_pair<OUT_DT>(y[2], y[3]),
+                                                       pack_pair<OUT_DT>(y[4], y[5]), pack_pair<OUT_DT>(y[6], y[7]));
+          }
         }
       }
     }
@@ -153,23 +160,15 @@ __device__ __forceinline__ void gemm_epilogue(const f32x16 (&acc)[FM][FN], int64
                                               const float *row_scale, const uint16_t *row_norms,
                                               const void *bias, int bias_dtype, const EpiFactors<FM> &pre,
                                               void *out, int out_dtype, unsigned char *lds) {
-  const int lane = tid & 63, r = lane & 31, grp = lane >> 5;
-  const bool fast = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
-  if (fast) {
-    if (out_dtype == OQ_BF16)
-      gemm_epilogue_lds<FM, FN, OQ_BF16>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds);
-    else if (out_dtype == OQ_F16)
-      gemm_epilogue_lds<FM, FN, OQ_F16>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds);
-    else
-      gemm_epilogue_lds<FM, FN, OQ_F32>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds);
-  } else {
-    if (out_dtype == OQ_BF16)
-      gemm_epilogue_scalar<FM, FN, OQ_BF16>(acc, m_tile + wm, n_tile + wn, r, grp, M, N, row_scale, row_norms, bias, bias_dtype, out);
-    else if (out_dtype == OQ_F16)
-      gemm_epilogue_scalar<FM, FN, OQ_F16>(acc, m_tile + wm, n_tile + wn, r, grp, M, N, row_scale, row_norms, bias, bias_dtype, out);
-    else
-      gemm_epilogue_scalar<FM, FN, OQ_F32>(acc, m_tile + wm, n_tile + wn, r, grp, M, N, row_scale, row_norms, bias, bias_dtype, out);
-  }
+  (void)row_scale; (void)row_norms; (void)bias; (void)bias_dtype;
+  const bool interior = m_tile + 64 * FM <= M && n_tile + tile_n <= N;  // uniform over the workgroup
+#define OQ_EPILOGUE_CASE(DT)                                                                                   \
+  if (interior) gemm_epilogue_typed<FM, FN, DT, false>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds); \
+  else gemm_epilogue_typed<FM, FN, DT, true>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds)
+  if (out_dtype == OQ_BF16) { OQ_EPILOGUE_CASE(OQ_BF16); }
+  else if (out_dtype == OQ_F16) { OQ_EPILOGUE_CASE(OQ_F16); }
+  else { OQ_EPILOGUE_CASE(OQ_F32); }
+#undef OQ_EPILOGUE_CASE
 }
 
 }  // namespace oq

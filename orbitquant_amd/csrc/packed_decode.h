@@ -82,26 +82,20 @@ __device__ __forceinline__ uint32_t lut_field(uint32_t base, uint32_t word, int 
   return lds_read_u32((__builtin_amdgcn_ubfe(word, pos, width) << (LR + 2)) + base);
 }
 
-// ---- weight decode: the dwords of one lane's 32-value run -> operand of MFMA q ----
+// ---- weight decode: the dwords of one lane's 32-value run -> dword p (two values) of the operand of MFMA q ----
 template <int BITS, int LR = 5>
-__device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint32_t base) {
-  uint32_t o[4];
+__device__ __forceinline__ uint32_t decode_w_piece(const uint32_t (&w)[BITS], int q, int p, uint32_t base) {
   if constexpr (BITS == 4) {
-    const uint32_t f = w[q];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 8 * p, 8);
+    return lut_field<LR>(base, w[q], 8 * p, 8);
   } else if constexpr (BITS == 2) {
-    const uint32_t f = w[q >> 1] >> (16 * (q & 1));
-#pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 4 * p, 4);
+    return lut_field<LR>(base, w[q >> 1], 16 * (q & 1) + 4 * p, 4);
   } else if constexpr (BITS == 3) {
     uint32_t f;
     if (q == 0) f = w[0];
     else if (q == 1) f = __builtin_amdgcn_alignbit(w[1], w[0], 24);
     else if (q == 2) f = __builtin_amdgcn_alignbit(w[2], w[1], 16);
     else f = w[2] >> 8;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) o[p] = lut_field<LR>(base, f, 6 * p, 6);
+    return lut_field<LR>(base, f, 6 * p, 6);
   } else if constexpr (BITS == 6) {
     // 48-bit field at bit 48q of six dwords: eight 6-bit codes
     uint32_t lo, hi;  // lo: codes 0..4 and two bits of code 5; hi: the rest
@@ -109,23 +103,21 @@ __device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint
     else if (q == 1) { lo = __builtin_amdgcn_alignbit(w[2], w[1], 16); hi = w[2] >> 16; }
     else if (q == 2) { lo = w[3]; hi = w[4]; }
     else { lo = __builtin_amdgcn_alignbit(w[5], w[4], 16); hi = w[5] >> 16; }
-    const uint32_t mid = __builtin_amdgcn_alignbit(hi, lo, 24);  // bits 24..55 of the field
-    const uint32_t c[8] = {lo & 63u, (lo >> 6) & 63u, (lo >> 12) & 63u, (lo >> 18) & 63u,
-                           mid & 63u, (mid >> 6) & 63u, (mid >> 12) & 63u, (mid >> 18) & 63u};
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-      o[p] = __builtin_amdgcn_perm(lut_at<LR>(base, c[2 * p + 1]), lut_at<LR>(base, c[2 * p]), 0x07060100u);
+    const uint32_t src = p < 2 ? lo : __builtin_amdgcn_alignbit(hi, lo, 24);  // codes 0..3 | codes 4..7
+    const uint32_t c0 = (src >> (12 * (p & 1))) & 63u, c1 = (src >> (12 * (p & 1) + 6)) & 63u;
+    return __builtin_amdgcn_perm(lut_at<LR>(base, c1), lut_at<LR>(base, c0), 0x07060100u);
   } else {  // 8 bits
-    const uint32_t lo = w[2 * q], hi = w[2 * q + 1];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const uint32_t src = p < 2 ? lo : hi;
-      const uint32_t e0 = lut_at<LR>(base, (src >> (16 * (p & 1))) & 0xffu);
-      const uint32_t e1 = lut_at<LR>(base, (src >> (16 * (p & 1) + 8)) & 0xffu);
-      o[p] = __builtin_amdgcn_perm(e1, e0, 0x07060100u);
-    }
+    const uint32_t src = p < 2 ? w[2 * q] : w[2 * q + 1];
+    const uint32_t e0 = lut_at<LR>(base, (src >> (16 * (p & 1))) & 0xffu);
+    const uint32_t e1 = lut_at<LR>(base, (src >> (16 * (p & 1) + 8)) & 0xffu);
+    return __builtin_amdgcn_perm(e1, e0, 0x07060100u);
   }
-  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+template <int BITS, int LR = 5>
+__device__ __forceinline__ uint4 decode_w(const uint32_t (&w)[BITS], int q, uint32_t base) {
+  return make_uint4(decode_w_piece<BITS, LR>(w, q, 0, base), decode_w_piece<BITS, LR>(w, q, 1, base),
+                    decode_w_piece<BITS, LR>(w, q, 2, base), decode_w_piece<BITS, LR>(w, q, 3, base));
 }
 
 // eight 4-bit activation codes (one dword) -> operand of one MFMA

@@ -1,13 +1,12 @@
-// Packed-weight GEMM on the gfx950 matrix cores.
+// Packed-weight GEMM on the gfx950 matrix cores: 4-bit activation codes x packed weight indices.
 //
-//   out[m,n] = (sum_k A[m,k] * c_w[idx[n,k]]) * scale[m] * r_w[n] + bias[n]
+//   out[m,n] = (sum_k c_a[code[m,k]] * c_w[idx[n,k]]) * scale[m] * r_w[n] + bias[n]
 //
-// A is either packed 4-bit activation codes (decoded through a codebook table)
-// or 16-bit float values; idx is the flat little-endian bit stream of 2/3/4/6/8
-// bit weight indices, read from HBM as it is stored.  Nothing is dequantized to
-// memory: every wavefront loads the packed dwords of its own rows straight into
-// registers, turns them into bf16 MFMA operands through lookup tables held in
-// LDS, and feeds v_mfma_f32_32x32x16_bf16.
+// code is the nibble stream of activation codes, idx the flat little-endian bit
+// stream of 2/3/4/6/8-bit weight indices, both read from HBM as they are stored.
+// Nothing is dequantized to memory: every wavefront loads the packed dwords of
+// its own rows straight into registers, turns them into bf16 MFMA operands
+// through lookup tables held in LDS, and feeds v_mfma_f32_32x32x16_bf16.
 //
 // Operand layout.  One MFMA consumes, per lane, eight k-values of one row
 // (lane l: row l%32, k-group l/32).  A dot product does not care in which order
@@ -17,18 +16,34 @@
 // which makes every global load of packed data one contiguous 4*bits-byte run
 // per lane (16 bytes for 4-bit), with no cross-lane shuffles and no LDS staging.
 //
-// Lookup tables: see packed_decode.h (pair tables, replicated per LDS bank).
+// Lookup tables.  One 64 KB block of LDS, 256 rows of 256 bytes, placed at LDS
+// address 0.  Row e holds, 32 times each, the dword of weight-table entry e
+// (bytes 0..127) and of activation-table entry e (bytes 128..255); lane l reads
+// copy l%32, so the lanes of a wavefront never collide on a bank whatever codes
+// they hold.  The activation table and the 4-bit weight table are indexed by a
+// whole byte of the packed stream (two codes) and return both bf16 values in one
+// dword, and because a row is 256 bytes the LDS address of a lookup is simply
+//   byte 0 = the lane's offset, byte 1 = the code byte
+// which one v_perm_b32 assembles: a lookup is one VALU instruction plus one
+// ds_read_b32 for two operand values.  Other weight widths index the same rows
+// with a bit-field extract (pair tables for 2/3 bits, single-code for 6/8).
+//
+// The instruction stream of a wavefront is what bounds this kernel (per MFMA of
+// 32 cycles it may issue about eight other instructions), hence the tile shapes:
+// a wavefront owning FM x FN tiles of 32x32 issues 4*(FM+FN) lookups per FM*FN MFMAs.
+#include <type_traits>
+
 #include "gemm_epilogue.h"
 
 namespace oq {
 namespace {
 
-enum AMode { A_NIBBLE = 0, A_BF16 = 1, A_F16 = 2 };
+enum AMode { A_NIBBLE = 0 };
 
 struct GemmArgs {
-  const uint8_t *a;          // [M, K/2] nibble codes or [M, K] 16-bit floats
+  const uint8_t *a;          // [M, K/2] nibble codes
   const float *row_scale;    // [M] or NULL
-  const float *act_cents;    // [16] (nibble mode)
+  const float *act_cents;    // [a_levels]
   int a_levels;
   const uint8_t *w;          // packed index stream
   const uint16_t *row_norms; // bf16 [N]
@@ -41,46 +56,50 @@ struct GemmArgs {
   int tiles_m, tiles_n;
 };
 
-template <int AM> struct ARaw { uint4 v[AM == A_NIBBLE ? 1 : 4]; };
+constexpr int kTableBytes = 65536;
+static_assert(kEpiLdsBytes <= kTableBytes, "the epilogue reuses the table block");
 
-template <int AM>
-__device__ __forceinline__ void load_a(const uint8_t *p, ARaw<AM> &r) {
-  const uint4 *q = reinterpret_cast<const uint4 *>(p);
-#pragma unroll
-  for (int i = 0; i < (AM == A_NIBBLE ? 1 : 4); ++i) r.v[i] = q[i];
+// dword of weight-table row e
+template <int BITS>
+__device__ __forceinline__ uint32_t w_table_entry(const float *cents, int e) {
+  constexpr int levels = 1 << BITS;
+  if constexpr (BITS <= 4) {
+    if (e >= levels * levels) return 0u;
+    return pack16(cents[e & (levels - 1)], cents[e >> BITS], false);
+  } else {
+    if (e >= levels) return 0u;
+    const float v = cents[e];
+    return pack16(v, v, false);
+  }
 }
 
-template <int AM>
-__device__ __forceinline__ f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
-  if constexpr (AM == A_F16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+// LDS address of the row selected by byte `p` of `word`: (byte << 8) | lane offset
+__device__ __forceinline__ uint32_t row_address(uint32_t word, uint32_t lane_off, int p) {
+  return __builtin_amdgcn_perm(word, lane_off, 0x03020400u + (static_cast<uint32_t>(p) << 8));
+}
+
+__device__ __forceinline__ uint4 decode_bytes(uint32_t f, uint32_t lane_off) {
+  return make_uint4(lds_read_u32(row_address(f, lane_off, 0)), lds_read_u32(row_address(f, lane_off, 1)),
+                    lds_read_u32(row_address(f, lane_off, 2)), lds_read_u32(row_address(f, lane_off, 3)));
 }
 
 // Workgroup = 4 wavefronts in a 2x2 arrangement; each wavefront owns FM x FN MFMA tiles of 32x32.
-template <int AM, int BITS, int FM, int FN>
+// NBUF = K-steps of packed operands held in registers (NBUF-1 of them in flight from memory).
+template <int AM, int BITS, int FM, int FN, int NBUF = (FM * FN >= 12 ? 2 : 3)>
 __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
-  extern __shared__ __align__(16) uint32_t lds[];
-  uint32_t *wlut = lds;
-  uint32_t *alut = lds + WLut<BITS>::kDwords;
+  __shared__ __attribute__((aligned(65536))) uint32_t lds[kTableBytes / 4];
 
-  // Loads of one wavefront return in order, so the handful of centroid values this thread
-  // needs for its table entries are requested first, then the packed operands of the first
-  // two K-steps; the tables are written while the packed data is still in flight.
-  constexpr int kWEntries = WLut<BITS>::kEntries;
-  float lut_w0 = 0.0f, lut_w1 = 0.0f, lut_a0 = 0.0f, lut_a1 = 0.0f;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, grp = lane >> 5;
+
+  // Loads of one wavefront return in order, so the centroid values this thread needs for its
+  // table row are requested first, then the packed operands of the first K-steps; the tables
+  // are written while the packed data is still in flight.
+  const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
+  uint32_t my_a;
   {
-    const int e = threadIdx.x;
-    if (e < kWEntries) {
-      lut_w0 = g.w_cents[WLut<BITS>::kPair ? (e & ((1 << BITS) - 1)) : e];
-      lut_w1 = g.w_cents[WLut<BITS>::kPair ? (e >> BITS) : e];
-    }
-    if constexpr (AM == A_NIBBLE) {
-      const int c0 = e & 15, c1 = e >> 4;
-      lut_a0 = c0 < g.a_levels ? g.act_cents[c0] : 0.0f;
-      lut_a1 = c1 < g.a_levels ? g.act_cents[c1] : 0.0f;
-    }
+    const int c0 = tid & 15, c1 = tid >> 4;
+    my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
   }
 
   constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
@@ -97,32 +116,52 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int pid_m = first_m + (bid % width) % gsz;
   const int pid_n = (bid % width) / gsz;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, grp = lane >> 5;
-  const uint32_t wbase = lds_byte_address(wlut) + 4 * r;
-  const uint32_t abase = lds_byte_address(alut) + 4 * r;
+  const uint32_t lds_base = lds_byte_address(lds);           // a multiple of 65536 by the alignment
+  const uint32_t w_off = lds_base + 4 * r, a_off = lds_base + 128 + 4 * r;  // the lane's copy inside a table row
   const int64_t m_base = static_cast<int64_t>(pid_m) * TM + (wave >> 1) * (FM * 32);
   const int64_t n_base = static_cast<int64_t>(pid_n) * TN + (wave & 1) * (FN * 32);
 
   EpiFactors<FM> epi;
   gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, (wave >> 1) * (FM * 32), TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
 
-  constexpr int A_ROW_STEP = AM == A_NIBBLE ? 32 : 128;  // bytes of one row consumed per K-step of 64
-  constexpr int A_GRP_OFF = AM == A_NIBBLE ? 16 : 64;
-  const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K * 2;
+  const int64_t a_row_bytes = g.K / 2;
   const int64_t w_row_bytes = g.K * BITS / 8;
-
   const uint8_t *ap[FM];
   const uint8_t *wp[FN];
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int64_t row = min(m_base + 32 * i + r, g.M - 1);
-    ap[i] = g.a + row * a_row_bytes + grp * A_GRP_OFF;
-  }
+  for (int i = 0; i < FM; ++i) ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * 16;
 #pragma unroll
-  for (int j = 0; j < FN; ++j) {
-    const int64_t row = min(n_base + 32 * j + r, g.N - 1);
-    wp[j] = g.w + row * w_row_bytes + grp * (4 * BITS);
+  for (int j = 0; j < FN; ++j) wp[j] = g.w + min(n_base + 32 * j + r, g.N - 1) * w_row_bytes + grp * (4 * BITS);
+
+  // packed operands of NBUF consecutive K-steps
+  uint4 pa[NBUF][FM];
+  uint32_t pw[NBUF][FN][BITS];
+  const int steps = static_cast<int>(g.K / 64);
+  // operand `e` (A row-tile e < FM, else weight column-tile e-FM) of K-step ks into buffer B
+  auto fetch_one = [&](auto buf, int e, int ks) {
+    constexpr int B = decltype(buf)::value;
+    const int64_t s = min(ks, steps - 1);  // past the end: re-read the last step (never multiplied)
+    if (e < FM) pa[B][e] = *reinterpret_cast<const uint4 *>(ap[e] + s * 32);
+    else load_w<BITS>(wp[e - FM] + s * (8 * BITS), pw[B][e - FM]);
+  };
+  auto fetch = [&](auto buf, int ks) {
+#pragma unroll
+    for (int e = 0; e < FM + FN; ++e) fetch_one(buf, e, ks);
+  };
+  // buffers 0..NBUF-2 <- K-steps 0..NBUF-2; K-step NBUF-1 is requested by the first step of the loop
+  fetch(std::integral_constant<int, 0>{}, 0);
+  if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
+
+  {  // tables: wavefront w writes rows 64w..64w+63, 16-byte chunk c of a row is a weight copy
+     // (c < 8) or an activation copy; lane l writes chunk l%16 of row 64w + 4i + l/16
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int src = 4 * i + (lane >> 4);
+      const uint32_t ew = __shfl(my_w, src), ea = __shfl(my_a, src);
+      const uint32_t d = (lane & 8) ? ea : ew;
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + (64 * wave + src) * 256 + (lane & 15) * 16) =
+          make_uint4(d, d, d, d);
+    }
   }
 
   f32x16 acc[FM][FN];
@@ -132,103 +171,91 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  // ---- main loop: software pipeline over "q-steps" (one MFMA k-slice of 16) -------
-  // While the matrix core works on the operands decoded for q-step t, the wavefront
-  // issues the table lookups for q-step t+1; packed dwords for K-step ks+1 are in
-  // flight from global memory during K-step ks.
-  ARaw<AM> a_cur[FM], a_nxt[FM];
-  uint32_t w_cur[FN][BITS], w_nxt[FN][BITS];
-#pragma unroll
-  for (int i = 0; i < FM; ++i) load_a<AM>(ap[i], a_cur[i]);
-#pragma unroll
-  for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j], w_cur[j]);
-
-  const int steps = static_cast<int>(g.K / 64);
-  if (steps > 1) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + A_ROW_STEP, a_nxt[i]);
-#pragma unroll
-    for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + 8 * BITS, w_nxt[j]);
-  }
-
-  {  // table entries: one per thread, 32 copies each
-    const int e = threadIdx.x;
-    if (e < kWEntries) {
-      const uint32_t d = pack16(lut_w0, lut_w1, AM == A_F16);
-      uint4 *dst = reinterpret_cast<uint4 *>(wlut + e * 32);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) dst[i] = make_uint4(d, d, d, d);
-    }
-    if constexpr (AM == A_NIBBLE) {
-      const uint32_t d = pack16(lut_a0, lut_a1, false);
-      uint4 *dst = reinterpret_cast<uint4 *>(alut + e * 32);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) dst[i] = make_uint4(d, d, d, d);
-    }
-  }
   __syncthreads();
 
-  auto decode = [&](int q, uint4 (&af)[FM], uint4 (&bf)[FN]) {
+  // ---- main loop: software pipeline over "phases" (one MFMA k-slice of 16) -------
+  // While the matrix core works on the operands looked up in the previous phase, the
+  // wavefront issues the table lookups for the next one.  The instruction order is fixed by
+  // hand: after every MFMA come kLook lookups (address arithmetic + LDS read), and nothing
+  // may be moved across the boundary between two such groups, so the matrix core never
+  // waits behind a burst of lookups and the LDS queue never runs dry.  The first phase of a
+  // K-step also carries the FM+FN global loads of the K-step NBUF-1 ahead, one per group.
+  constexpr int kLookups = 4 * (FM + FN), kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
+  constexpr int kLook = (kLookups + kGroups - 1) / kGroups;
+  uint32_t oa[2][FM][4], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
+
+  // lookup t of a phase, in the order the MFMAs of the next phase want their operands:
+  // A tile 0, every weight tile, then A tiles 1..FM-1.  Split in two halves so that the
+  // address of a lookup is computed one group before its LDS read is issued.
+  auto lookup_address = [&](auto buf, int q, int t) -> uint32_t {
+    constexpr int B = decltype(buf)::value;
+    const int p = t & 3, f = t >> 2;
+    if (f == 0 || f > FN) {
+      const int i = f == 0 ? 0 : f - FN;
+      const uint32_t word = q == 0 ? pa[B][i].x : q == 1 ? pa[B][i].y : q == 2 ? pa[B][i].z : pa[B][i].w;
+      return row_address(word, a_off, p);
+    }
+    if constexpr (BITS == 4) return row_address(pw[B][f - 1][q], w_off, p);
+    else return 0u;
+  };
+  auto lookup_read = [&](auto buf, int q, int set, int t, uint32_t address) {
+    constexpr int B = decltype(buf)::value;
+    const int p = t & 3, f = t >> 2;
+    if (f == 0 || f > FN) {
+      oa[set][f == 0 ? 0 : f - FN][p] = lds_read_u32(address);
+    } else {
+      if constexpr (BITS == 4) ob[set][f - 1][p] = lds_read_u32(address);
+      else ob[set][f - 1][p] = decode_w_piece<BITS, 6>(pw[B][f - 1], q, p, w_off);
+    }
+  };
+  // lookups of (buf, q) into `set` interleaved with the MFMAs on the other set
+  auto phase = [&](auto buf, int q, int set, auto fetch_buf, int fetch_ks, bool with_fetch) {
+    uint32_t addr[2][kLook];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      if constexpr (AM == A_NIBBLE) {
-        const uint32_t f = q == 0 ? a_cur[i].v[0].x : q == 1 ? a_cur[i].v[0].y : q == 2 ? a_cur[i].v[0].z : a_cur[i].v[0].w;
-        af[i] = decode_a_nibble(f, abase);
-      } else {
-        af[i] = a_cur[i].v[q];
+    for (int t = 0; t < kLookups / kGroups; ++t) addr[0][t] = lookup_address(buf, q, t);
+#pragma unroll
+    for (int m = 0; m < kGroups; ++m) {
+      const int i = m / FN, j = m % FN;
+      const int lo = m * kLookups / kGroups, hi = (m + 1) * kLookups / kGroups, hi2 = (m + 2) * kLookups / kGroups;
+      if (with_fetch && m < FM + FN) fetch_one(fetch_buf, m, fetch_ks);
+      const uint4 bw = make_uint4(ob[set ^ 1][j][0], ob[set ^ 1][j][1], ob[set ^ 1][j][2], ob[set ^ 1][j][3]);
+      const uint4 av = make_uint4(oa[set ^ 1][i][0], oa[set ^ 1][i][1], oa[set ^ 1][i][2], oa[set ^ 1][i][3]);
+      // weights first: the accumulator tile is the transposed output tile
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, av),
+                                                          acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int t = lo; t < hi; ++t) lookup_read(buf, q, set, t, addr[m & 1][t - lo]);
+      if (m + 1 < kGroups) {
+#pragma unroll
+        for (int t = hi; t < hi2; ++t) addr[(m + 1) & 1][t - hi] = lookup_address(buf, q, t);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int j = 0; j < FN; ++j) bf[j] = decode_w<BITS>(w_cur[j], q, wbase);
   };
-  auto multiply = [&](const uint4 (&af)[FM], const uint4 (&bf)[FN]) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j) acc[i][j] = mfma<AM>(bf[j], af[i], acc[i][j]);  // weights first: transposed tile
-  };
-  // interleave hint: after each MFMA, the lookups' address arithmetic and LDS reads
-  constexpr int kLookupsPerMfma = (AM == A_NIBBLE ? (FM + FN) : FN) * 4 / (FM * FN);
-  auto interleave = [&]() {
-#if defined(OQ_SCHED_HINTS)
-#pragma unroll
-    for (int i = 0; i < FM * FN; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2 * kLookupsPerMfma, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, kLookupsPerMfma, 0);
-    }
-#endif
+  // one K-step out of buffer B; its last phase looks up the first operands of buffer B+1
+  auto step = [&](auto buf, int ks) {
+    constexpr int B = decltype(buf)::value;
+    constexpr auto prev = std::integral_constant<int, (B + NBUF - 1) % NBUF>{};
+    constexpr auto next = std::integral_constant<int, (B + 1) % NBUF>{};
+    phase(buf, 1, 1, prev, ks + NBUF - 1, FM + FN <= FM * FN);
+    if constexpr (FM + FN > FM * FN) fetch(prev, ks + NBUF - 1);
+    phase(buf, 2, 0, prev, 0, false);
+    phase(buf, 3, 1, prev, 0, false);
+    phase(next, 0, 0, prev, 0, false);
   };
 
-  uint4 af0[FM], bf0[FN], af1[FM], bf1[FN];
-  decode(0, af0, bf0);
-  for (int ks = 0; ks < steps; ++ks) {
-    decode(1, af1, bf1);
-    multiply(af0, bf0);
-    interleave();
-    decode(2, af0, bf0);
-    multiply(af1, bf1);
-    interleave();
-    decode(3, af1, bf1);
-    multiply(af0, bf0);
-    interleave();
-    // rotate: K-step ks+1 becomes current, K-step ks+2 goes in flight
 #pragma unroll
-    for (int i = 0; i < FM; ++i) a_cur[i] = a_nxt[i];
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int d = 0; d < BITS; ++d) w_cur[j][d] = w_nxt[j][d];
-    if (ks + 2 < steps) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i) load_a<AM>(ap[i] + static_cast<int64_t>(ks + 2) * A_ROW_STEP, a_nxt[i]);
-#pragma unroll
-      for (int j = 0; j < FN; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(ks + 2) * (8 * BITS), w_nxt[j]);
-    }
-    decode(0, af0, bf0);  // of K-step ks+1 (unused after the last step)
-    multiply(af1, bf1);
-    interleave();
+  for (int t = 0; t < 4 * (FM + FN); ++t)
+    lookup_read(std::integral_constant<int, 0>{}, 0, 0, t, lookup_address(std::integral_constant<int, 0>{}, 0, t));
+  int ks = 0;
+  for (; ks + NBUF <= steps; ks += NBUF) {
+    step(std::integral_constant<int, 0>{}, ks);
+    step(std::integral_constant<int, 1>{}, ks + 1);
+    if constexpr (NBUF == 3) step(std::integral_constant<int, 2>{}, ks + 2);
+  }
+  if (ks < steps) {
+    step(std::integral_constant<int, 0>{}, ks);
+    if (NBUF == 3 && ks + 1 < steps) step(std::integral_constant<int, 1>{}, ks + 1);
   }
 
   __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused by the epilogue
@@ -244,20 +271,14 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  size_t smem = (WLut<BITS>::kDwords + (AM == A_NIBBLE ? kALutDwords : 0)) * sizeof(uint32_t);
-  if (smem < static_cast<size_t>(kEpiLdsBytes)) smem = kEpiLdsBytes;  // the epilogue reuses LDS
   auto kern = packed_gemm_kernel<AM, BITS, FM, FN>;
-  if (smem > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(smem)) != hipSuccess)
-      return fail(OQ_ERR_LAUNCH, "packed_gemm: cannot reserve %zu bytes of LDS", smem);
-  }
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), smem, stream, g);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), 0, stream, g);
   return check_launch("packed_gemm");
 }
 
 template <int AM, int BITS>
 int launch_bits(const GemmArgs &g, int tile, hipStream_t stream) {
+  if (tile == 3) return launch_cfg<AM, BITS, 4, 3>(g, stream);
   if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
   if (tile == 1) return launch_cfg<AM, BITS, 2, 4>(g, stream);
   return launch_cfg<AM, BITS, 2, 2>(g, stream);
@@ -280,7 +301,7 @@ int launch_mode(const GemmArgs &g, int bits, int tile, hipStream_t stream) {
 // Tile choice: the largest tile that still gives every CU work.
 int gemm_choose_tile(int64_t M, int64_t N) {
   const char *force = getenv("OQ_GEMM_TILE");
-  if (force != nullptr && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
+  if (force != nullptr && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
   auto tiles = [&](int tm, int tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
   if (tiles(256, 256) >= 512) return 2;
   if (tiles(128, 256) >= 384) return 1;

@@ -90,18 +90,10 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint32_t f = q == 0 ? bt.a[d].x : q == 1 ? bt.a[d].y : q == 2 ? bt.a[d].z : bt.a[d].w;
-#if defined(OQ_EXP_NOADECODE) || defined(OQ_EXP_NODECODE)
-          const uint4 af = make_uint4(f, f, f, f);
-#else
           const uint4 af = decode_a_nibble<kLR>(f, abase);
-#endif
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-#if defined(OQ_EXP_NODECODE)
-            const uint4 bf = make_uint4(bt.w[d][j][0], bt.w[d][j][1 % BITS], bt.w[d][j][BITS - 1], bt.w[d][j][0]);
-#else
             const uint4 bf = decode_w<BITS, kLR>(bt.w[d][j], q, wbase);
-#endif
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
                                                              __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
           }

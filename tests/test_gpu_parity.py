@@ -253,7 +253,7 @@ def test_packed_linear_tile_kernel(dev, m, n, k, wbits, abits, block, with_bias,
     check_outputs(got_u8.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "u8")
 
 
-@pytest.mark.parametrize("tile", ["0", "1", "2"])
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3"])
 def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
     monkeypatch.setenv("OQ_GEMM_TILE", tile)
     rng = np.random.default_rng(int(tile) + 50)
