@@ -31,7 +31,6 @@ SOURCES = {
     "rotate_quantize.hip": ["-ffp-contract=off"],
     "packed_generic.hip": [],
     "packed_gemm.hip": [],
-    "packed_gemm_staged.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
 }

@@ -52,12 +52,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream);
-int gemm_choose_tile(int64_t M, int64_t N);
-bool gemm_staged_supported(int64_t K, int bits);
-int gemm_staged_dispatch(const void *codes, const float *row_scale, const float *act_cents, int a_levels,
-                         const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
-                         const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                         int out_dtype, int tile, hipStream_t stream);
+int gemm_choose_tile(int64_t M, int64_t N, int64_t K);
 bool gemm_av_supported(int64_t K, int bits);
 int gemm_av_dispatch(bool f16, const void *a, const float *row_scale, const uint8_t *w, int bits,
                      const uint16_t *row_norms, const float *w_cents, const void *bias, int bias_dtype,
@@ -129,9 +124,6 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
   if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
     return gemv_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
-  if (fast_ptrs && tiled_out && code_format == OQ_CODES_NIBBLE && gemm_staged_supported(K, w_bits) && getenv("OQ_GEMM_STAGED") != nullptr)
-    return gemm_staged_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
-                                bias, bias_dtype, M, N, K, out, out_dtype, gemm_choose_tile(M, N), s);
   if (fast_ptrs && tiled_out && code_format == OQ_CODES_NIBBLE && gemm_supported(K, w_bits))
     return gemm_dispatch(0, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
@@ -149,7 +141,7 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   hipStream_t s = as_stream(stream);
   if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
     return gemm_av_dispatch(x_dtype == OQ_F16, x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype,
-                            M, N, K, out, out_dtype, gemm_choose_tile(M, N), s);
+                            M, N, K, out, out_dtype, gemm_choose_tile(M, N, K), s);
   return generic_matmul_float(x, x_dtype, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N,
                               K, out, out_dtype, s);
 }

@@ -159,9 +159,9 @@ __device__ __forceinline__ void gemm_epilogue(const f32x16 (&acc)[FM][FN], int64
                                               int wn, int tile_n, int tid, int64_t M, int64_t N,
                                               const float *row_scale, const uint16_t *row_norms,
                                               const void *bias, int bias_dtype, const EpiFactors<FM> &pre,
-                                              void *out, int out_dtype, unsigned char *lds) {
+                                              void *out, int out_dtype, unsigned char *lds, int tile_m = 64 * FM) {
   (void)row_scale; (void)row_norms; (void)bias; (void)bias_dtype;
-  const bool interior = m_tile + 64 * FM <= M && n_tile + tile_n <= N;  // uniform over the workgroup
+  const bool interior = m_tile + tile_m <= M && n_tile + tile_n <= N;  // uniform over the workgroup
 #define OQ_EPILOGUE_CASE(DT)                                                                                   \
   if (interior) gemm_epilogue_typed<FM, FN, DT, false>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds); \
   else gemm_epilogue_typed<FM, FN, DT, true>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds)

@@ -83,10 +83,16 @@ __device__ __forceinline__ uint4 decode_bytes(uint32_t f, uint32_t lane_off) {
                     lds_read_u32(row_address(f, lane_off, 2)), lds_read_u32(row_address(f, lane_off, 3)));
 }
 
-// Workgroup = 4 wavefronts in a 2x2 arrangement; each wavefront owns FM x FN MFMA tiles of 32x32.
+// Workgroup = 4 wavefronts; each wavefront owns FM x FN MFMA tiles of 32x32.
+//   KSPLIT = 1: the wavefronts sit 2x2 on a [64 FM x 64 FN] output tile, each runs over all of K.
+//   KSPLIT = 4: all four work on the SAME [32 FM x 32 FN] output tile, each over a quarter of K
+//               (for short-and-wide problems whose output has too few tiles to fill the chip);
+//               the partial tiles are then summed through LDS in a fixed order, each wavefront
+//               ending up with one 32-row slice of the tile, which it scales and stores.  FM = 4.
 // NBUF = K-steps of packed operands held in registers (NBUF-1 of them in flight from memory).
-template <int AM, int BITS, int FM, int FN, int NBUF = (FM * FN >= 12 ? 2 : 3)>
+template <int AM, int BITS, int FM, int FN, int KSPLIT = 1, int NBUF = (FM * FN >= 12 ? 2 : 3)>
 __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
+  static_assert(KSPLIT == 1 || (KSPLIT == 4 && FM == 4), "K split: four wavefronts, four row slices");
   __shared__ __attribute__((aligned(65536))) uint32_t lds[kTableBytes / 4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
   }
 
-  constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
+  constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
   // tile order: spread consecutive workgroup ids over the 8 XCDs' private L2s in
   // contiguous chunks, then walk groups of 4 tile-rows column by column
   int bid = blockIdx.x;
@@ -118,11 +124,12 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 
   const uint32_t lds_base = lds_byte_address(lds);           // a multiple of 65536 by the alignment
   const uint32_t w_off = lds_base + 4 * r, a_off = lds_base + 128 + 4 * r;  // the lane's copy inside a table row
-  const int64_t m_base = static_cast<int64_t>(pid_m) * TM + (wave >> 1) * (FM * 32);
-  const int64_t n_base = static_cast<int64_t>(pid_n) * TN + (wave & 1) * (FN * 32);
+  const int wm = KSPLIT == 1 ? (wave >> 1) * (FM * 32) : 0, wn = KSPLIT == 1 ? (wave & 1) * (FN * 32) : 0;
+  const int64_t m_base = static_cast<int64_t>(pid_m) * TM + wm;
+  const int64_t n_base = static_cast<int64_t>(pid_n) * TN + wn;
 
   EpiFactors<FM> epi;
-  gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, (wave >> 1) * (FM * 32), TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+  gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
 
   const int64_t a_row_bytes = g.K / 2;
   const int64_t w_row_bytes = g.K * BITS / 8;
@@ -136,7 +143,13 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // packed operands of NBUF consecutive K-steps
   uint4 pa[NBUF][FM];
   uint32_t pw[NBUF][FN][BITS];
-  const int steps = static_cast<int>(g.K / 64);
+  const int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
+  if constexpr (KSPLIT > 1) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * 32;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) wp[j] += static_cast<int64_t>(wave) * steps * (8 * BITS);
+  }
   // operand `e` (A row-tile e < FM, else weight column-tile e-FM) of K-step ks into buffer B
   auto fetch_one = [&](auto buf, int e, int ks) {
     constexpr int B = decltype(buf)::value;
@@ -258,26 +271,71 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     if (NBUF == 3 && ks + 1 < steps) step(std::integral_constant<int, 1>{}, ks + 1);
   }
 
-  __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused by the epilogue
-  gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, (wave >> 1) * (FM * 32),
-                        (wave & 1) * (FN * 32), TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
-                        g.out_dtype, reinterpret_cast<unsigned char *>(lds));
+  __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused from here on
+  if constexpr (KSPLIT == 1) {
+    gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, wn, TN, tid, g.M, g.N,
+                          g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out, g.out_dtype,
+                          reinterpret_cast<unsigned char *>(lds));
+  } else {
+    // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
+    // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
+    // its own slice w.  Slot of destination s: [FN tiles][4 runs][64 lanes] of float4.
+    float4 *slots = reinterpret_cast<float4 *>(lds);
+    auto finish = [&](auto wt) {
+      constexpr int W = decltype(wt)::value;
+#pragma unroll
+      for (int d = 1; d < 4; ++d) {
+        const int dst = (W + d) & 3;
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4)
+            slots[((dst * FN + j) * 4 + a4) * 64 + lane] = make_float4(acc[dst][j][4 * a4 + 0], acc[dst][j][4 * a4 + 1],
+                                                                       acc[dst][j][4 * a4 + 2], acc[dst][j][4 * a4 + 3]);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            const float4 v = slots[((W * FN + j) * 4 + a4) * 64 + lane];
+            acc[W][j][4 * a4 + 0] += v.x;
+            acc[W][j][4 * a4 + 1] += v.y;
+            acc[W][j][4 * a4 + 2] += v.z;
+            acc[W][j][4 * a4 + 3] += v.w;
+          }
+        __syncthreads();
+      }
+      EpiFactors<1> mine;
+      mine.rn = epi.rn;
+      mine.bv = epi.bv;
+      mine.sc[0] = epi.sc[W];
+      const f32x16 (&slice)[1][FN] = *reinterpret_cast<const f32x16 (*)[1][FN]>(&acc[W]);
+      gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * W, 0, TN, tid, g.M,
+                           g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
+                           reinterpret_cast<unsigned char *>(lds), TM);
+    };
+    if (wave == 0) finish(std::integral_constant<int, 0>{});
+    else if (wave == 1) finish(std::integral_constant<int, 1>{});
+    else if (wave == 2) finish(std::integral_constant<int, 2>{});
+    else finish(std::integral_constant<int, 3>{});
+  }
 }
 
-template <int AM, int BITS, int FM, int FN>
+template <int AM, int BITS, int FM, int FN, int KSPLIT = 1>
 int launch_cfg(GemmArgs g, hipStream_t stream) {
-  constexpr int TM = 2 * FM * 32, TN = 2 * FN * 32;
+  constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
   g.tiles_m = static_cast<int>((g.M + TM - 1) / TM);
   g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  auto kern = packed_gemm_kernel<AM, BITS, FM, FN>;
+  auto kern = packed_gemm_kernel<AM, BITS, FM, FN, KSPLIT>;
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), 0, stream, g);
   return check_launch("packed_gemm");
 }
 
 template <int AM, int BITS>
 int launch_bits(const GemmArgs &g, int tile, hipStream_t stream) {
+  if (tile == 4) return launch_cfg<AM, BITS, 4, 3, 4>(g, stream);
   if (tile == 3) return launch_cfg<AM, BITS, 4, 3>(g, stream);
   if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
   if (tile == 1) return launch_cfg<AM, BITS, 2, 4>(g, stream);
@@ -298,14 +356,40 @@ int launch_mode(const GemmArgs &g, int bits, int tile, hipStream_t stream) {
 
 }  // namespace
 
-// Tile choice: the largest tile that still gives every CU work.
-int gemm_choose_tile(int64_t M, int64_t N) {
+// Tile choice by a small cost model: a launch runs in `rounds` of as many workgroups as fit
+// on the chip at once; a workgroup costs a fixed prologue + epilogue and a time per K-step
+// of 64 (both measured on an MI355X, microseconds).  128x128 tiles fit two to a CU.
+int gemm_choose_tile(int64_t M, int64_t N, int64_t K) {
   const char *force = getenv("OQ_GEMM_TILE");
+  const bool can_split = K % 256 == 0;  // a quarter of the K-steps per wavefront
   if (force != nullptr && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
-  auto tiles = [&](int tm, int tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
-  if (tiles(256, 256) >= 512) return 2;
-  if (tiles(128, 256) >= 384) return 1;
-  return 0;
+  if (force != nullptr && force[0] == '4' && can_split) return 4;
+  struct Shape { int tm, tn; double fixed, per_step; };
+  static const Shape shapes[4] = {{128, 128, 4.5, 0.8}, {128, 256, 5.5, 1.0}, {256, 256, 7.0, 1.5}, {256, 192, 6.0, 1.15}};
+  const double steps = static_cast<double>(K / 64);
+  int best = 0;
+  double best_cost = 0.0;
+  for (int t = 0; t < 4; ++t) {
+    const int64_t tiles = ((M + shapes[t].tm - 1) / shapes[t].tm) * ((N + shapes[t].tn - 1) / shapes[t].tn);
+    double per_step = shapes[t].per_step;
+    int64_t capacity = 256;
+    if (t == 0) {
+      if (tiles <= 256) per_step = 0.5;  // one workgroup per CU: no LDS contention
+      else capacity = 512;
+    }
+    const double rounds = static_cast<double>((tiles + capacity - 1) / capacity);
+    const double cost = rounds * (shapes[t].fixed + steps * per_step);
+    if (t == 0 || cost < best_cost) {
+      best = t;
+      best_cost = cost;
+    }
+  }
+  if (can_split) {  // 128x96 tiles, four wavefronts share the K range (+ about 1.5 us of reduction)
+    const int64_t tiles = ((M + 127) / 128) * ((N + 95) / 96);
+    const double cost = static_cast<double>((tiles + 255) / 256) * (7.5 + steps / 4.0 * 1.15);
+    if (cost < best_cost) best = 4;
+  }
+  return best;
 }
 
 bool gemm_supported(int64_t K, int bits) {
@@ -321,7 +405,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
-  const int tile = gemm_choose_tile(M, N);
+  const int tile = gemm_choose_tile(M, N, K);
   if (a_mode != A_NIBBLE) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
   return launch_mode<A_NIBBLE>(g, bits, tile, stream);
 }

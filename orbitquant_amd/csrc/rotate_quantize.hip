@@ -1,12 +1,14 @@
 // Fused RPBH rotate + per-token Lloyd-Max quantize for gfx950.
 //
-// One 256-thread workgroup per token row.  The row is staged once in LDS as
+// One workgroup per token row: 256 threads, or fewer wavefronts when the row is shorter
+// than 1536 elements (a wavefront covers 512).  The row is staged once in LDS as
 // fp32 (coalesced 16-byte global loads), the sum of squares is taken in the
 // fixed order the C header documents, then every thread gathers eight
 // consecutive rotated slots from LDS (permutation), divides by (norm + eps),
 // applies the sign and runs the Walsh-Hadamard butterflies:
 //   distance 1,2,4        in registers (the thread's own eight values)
-//   distance 8 .. 256     across the lanes of the wavefront (lane xor 1 .. 32)
+//   distance 8 .. 256     across the lanes of the wavefront (lane xor 1 .. 32: DPP lane
+//                         exchanges up to 8, wavefront shuffles for 16 and 32)
 //   distance 512 ..       through LDS, regrouped so the stages are register-local
 // Every butterfly output is one fp32 add or subtract of two values of the
 // previous stage, so the result does not depend on this schedule.
@@ -14,6 +16,10 @@
 // This file must be compiled without FMA contraction: every fp32 operation
 // rounds once, exactly like the CPU statement of the algorithm.
 #pragma clang fp contract(off)
+
+#include <stdlib.h>
+
+#include <type_traits>
 
 #include "oq_common.h"
 
@@ -151,24 +157,95 @@ __device__ __forceinline__ void fwht_regs(float (&v)[N], int limit) {
   }
 }
 
+// Lane exchanges for the butterflies between lanes l and l xor J: DPP quad permutes (1, 2),
+// masked row shifts (4), a row rotate (8); wavefront shuffles for 16 and 32.
+__device__ __forceinline__ float dpp_xor1(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_xor2(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_xor4(float v) {
+  const int i = __builtin_bit_cast(int, v);
+  int o = __builtin_amdgcn_update_dpp(i, i, 0x104, 0xF, 0x5, false);  // lanes 0-3, 8-11 of a row <- lane + 4
+  o = __builtin_amdgcn_update_dpp(o, i, 0x114, 0xF, 0xA, false);      // lanes 4-7, 12-15 <- lane - 4
+  return __builtin_bit_cast(float, o);
+}
+__device__ __forceinline__ float dpp_xor8(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true));
+}
+template <int J>
+__device__ __forceinline__ float lane_xor(float v) {
+  if constexpr (J == 1) return dpp_xor1(v);
+  else if constexpr (J == 2) return dpp_xor2(v);
+  else if constexpr (J == 4) return dpp_xor4(v);
+  else if constexpr (J == 8) return dpp_xor8(v);
+  else return __shfl_xor(v, J, 64);
+}
+
+// x / (s + eps) is evaluated as q0 = x*r, then two residual corrections
+// q <- fma(fma(-q, d, x), r, q) with r = 1/d correctly rounded: the first makes q a
+// faithful quotient, the second rounds it correctly (Markstein), which is what the
+// IEEE division of the specification returns.  Inputs for which a residual could
+// underflow, or that are not finite, take the plain division instead.
+__device__ __forceinline__ float divide_by_row_norm(float x, float d, float r) {
+  float q = x * r;
+  q = __builtin_fmaf(__builtin_fmaf(-q, d, x), r, q);
+  q = __builtin_fmaf(__builtin_fmaf(-q, d, x), r, q);
+  return q;
+}
+__device__ __forceinline__ bool needs_plain_division(float x) {
+  const float ax = __builtin_fabsf(x);
+  return !((ax > 1e-30f || ax == 0.0f) && ax < 1e30f);
+}
+
+// Where the row is staged in LDS: 16-bit inputs stay 16-bit (half the LDS, so twice the rows
+// in flight per CU) unless the big-block path needs the buffer for fp32 intermediates.
+template <int DT, bool VEC, int LOG_G> struct RqStage {
+  static constexpr bool k16 = VEC && DT != OQ_F32 && LOG_G == 0;
+  static constexpr int kBytes = k16 ? 2 : 4;
+};
+
+struct PermSigns {
+  int4 pa, pb;
+  uint2 sg;
+};
+__device__ __forceinline__ void load_perm_signs(const RqArgs &a, int64_t c0, PermSigns &ps) {
+  if (c0 + kChunk <= a.K) {
+    ps.pa = *reinterpret_cast<const int4 *>(a.perm + c0);
+    ps.pb = *reinterpret_cast<const int4 *>(a.perm + c0 + 4);
+    ps.sg = *reinterpret_cast<const uint2 *>(a.signs + c0);
+  }
+}
+
 template <int DT, bool VEC, int LOG_G>
 __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
+  using Stage = RqStage<DT, VEC, LOG_G>;
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = t >> 6;
   const int64_t row = blockIdx.x;
   const int64_t K = a.K;
   const int Kp = a.passes * kPass;
-  float *xbuf = reinterpret_cast<float *>(smem);
-  float *bnd = xbuf + Kp;        // 256 floats
-  float *cent = bnd + 256;       // 256 floats
-  float *red = cent + 256;       // 4 floats (+ pad to 16 B)
-  uint8_t *cbuf = reinterpret_cast<uint8_t *>(red + 4);  // Kp bytes, big-block path only
+  float *bnd = reinterpret_cast<float *>(smem);  // 256 floats
+  float *cent = bnd + 256;                       // 256 floats
+  float *red = cent + 256;                       // 4 floats
+  float *xbuf = red + 4;                         // Kp elements of Stage::kBytes
+  uint16_t *xbuf16 = reinterpret_cast<uint16_t *>(xbuf);
+  uint8_t *cbuf = reinterpret_cast<uint8_t *>(xbuf) + static_cast<size_t>(Kp) * Stage::kBytes;  // Kp bytes, big-block path only
+
+  // Permutation and signs of the first pass: requested before anything else so their latency
+  // overlaps the row load (loads of one wavefront return in order).
+  PermSigns ps_cur, ps_nxt;
+  if constexpr (VEC) load_perm_signs(a, static_cast<int64_t>(t) * kChunk, ps_cur);
 
   // tables
-  bnd[t] = (t < a.levels - 1) ? a.bounds[t] : __builtin_inff();
-  cent[t] = (a.cents != nullptr && t < a.levels) ? a.cents[t] : 0.0f;
+  const int nthreads = blockDim.x;  // 64 * (wavefronts that own a part of the row), at most 256
+  for (int i = t; i < 256; i += nthreads) {
+    bnd[i] = (i < a.levels - 1) ? a.bounds[i] : __builtin_inff();
+    cent[i] = (a.cents != nullptr && i < a.levels) ? a.cents[i] : 0.0f;
+  }
 
   // ---- phase A: stage the row, sum of squares in the documented order --------
   const int64_t row_base = row * K;
@@ -176,24 +253,57 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   for (int p = 0; p < a.passes; ++p) {
     const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
     float f[kChunk];
-    load_chunk<DT, VEC>(a.x, row_base, i0, K, f);
-    float4 *dst = reinterpret_cast<float4 *>(xbuf + i0);
-    dst[0] = make_float4(f[0], f[1], f[2], f[3]);
-    dst[1] = make_float4(f[4], f[5], f[6], f[7]);
+    if constexpr (Stage::k16) {
+      uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+      if (i0 + kChunk <= K) raw = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(a.x) + row_base + i0);
+      *reinterpret_cast<uint4 *>(xbuf16 + i0) = raw;
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (DT == OQ_BF16) {
+          f[2 * j] = __uint_as_float(w[j] << 16);
+          f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        } else {
+          f[2 * j] = f16_bits_to_f32(static_cast<uint16_t>(w[j] & 0xffffu));
+          f[2 * j + 1] = f16_bits_to_f32(static_cast<uint16_t>(w[j] >> 16));
+        }
+      }
+    } else {
+      load_chunk<DT, VEC>(a.x, row_base, i0, K, f);
+      float4 *dst = reinterpret_cast<float4 *>(xbuf + i0);
+      dst[0] = make_float4(f[0], f[1], f[2], f[3]);
+      dst[1] = make_float4(f[4], f[5], f[6], f[7]);
+    }
     float s[kChunk];
 #pragma unroll
     for (int e = 0; e < kChunk; ++e) s[e] = f[e] * f[e];
     const float v8 = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
     q = (p == 0) ? v8 : q + v8;
   }
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) q = q + __shfl_xor(q, off, 64);
+  q = q + lane_xor<1>(q);
+  q = q + lane_xor<2>(q);
+  q = q + lane_xor<4>(q);
+  q = q + lane_xor<8>(q);
+  q = q + lane_xor<16>(q);
+  q = q + lane_xor<32>(q);
   if (lane == 0) red[wave] = q;
   __syncthreads();
-  const float total = (red[0] + red[1]) + (red[2] + red[3]);
+  const int nwaves = nthreads >> 6;  // wavefronts that were not launched own only padding: their sum is 0
+  const float total = (red[0] + (nwaves > 1 ? red[1] : 0.0f)) + ((nwaves > 2 ? red[2] : 0.0f) + (nwaves > 3 ? red[3] : 0.0f));
   const float s_norm = sqrtf(total);  // IEEE-rounded (hipcc's default for fp32 sqrt and division)
   const float denom = s_norm + a.eps;
+  const float recip = 1.0f / denom;
+  const bool row_plain = !(denom > 1e-30f && denom < 1e30f);  // the reciprocal itself would lose bits
   if (t == 0 && a.norms != nullptr) a.norms[row] = s_norm;
+
+  auto staged = [&](int i) -> float {
+    if constexpr (Stage::k16) {
+      if constexpr (DT == OQ_BF16) return bf16_bits_to_f32(xbuf16[i]);
+      else return f16_bits_to_f32(xbuf16[i]);
+    } else {
+      return xbuf[i];
+    }
+  };
 
   // ---- phase B: gather, divide, sign, butterflies up to distance 256 ----------
   const int h = a.block;
@@ -205,36 +315,54 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
     if (p < a.passes) {
       const int64_t c0 = static_cast<int64_t>(p) * kPass + t * kChunk;
       float y[kChunk];
+      if constexpr (VEC) {
+        if (p + 1 < a.passes) load_perm_signs(a, c0 + kPass, ps_nxt);  // one pass ahead
+      }
       if (VEC && c0 + kChunk <= K) {
-        const int4 pa = *reinterpret_cast<const int4 *>(a.perm + c0);
-        const int4 pb = *reinterpret_cast<const int4 *>(a.perm + c0 + 4);
-        const int idx[kChunk] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
-        const uint2 sg = *reinterpret_cast<const uint2 *>(a.signs + c0);
+        const int idx[kChunk] = {ps_cur.pa.x, ps_cur.pa.y, ps_cur.pa.z, ps_cur.pa.w,
+                                 ps_cur.pb.x, ps_cur.pb.y, ps_cur.pb.z, ps_cur.pb.w};
+        const uint2 sg = ps_cur.sg;
+        float xv[kChunk];
+        bool plain = row_plain;
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
+          xv[e] = staged(idx[e]);
+          plain = plain || needs_plain_division(xv[e]);
+          y[e] = divide_by_row_norm(xv[e], denom, recip);
+        }
+        if (__builtin_amdgcn_ballot_w64(plain) != 0) {  // rare, and uniform over the wavefront
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) y[e] = xv[e] / denom;
+        }
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) {  // multiply by the sign (+1 / -1 = 0xff): flip the sign bit
           const uint32_t sw = e < 4 ? sg.x : sg.y;
-          const float sign = static_cast<float>(static_cast<int8_t>((sw >> (8 * (e & 3))) & 0xff));
-          y[e] = (xbuf[idx[e]] / denom) * sign;
+          y[e] = __uint_as_float(__float_as_uint(y[e]) ^ ((sw << (24 - 8 * (e & 3))) & 0x80000000u));
         }
       } else {
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
-          if (c0 + e < K) y[e] = (xbuf[a.perm[c0 + e]] / denom) * static_cast<float>(a.signs[c0 + e]);
+          if (c0 + e < K) y[e] = (staged(a.perm[c0 + e]) / denom) * static_cast<float>(a.signs[c0 + e]);
           else y[e] = 0.0f;
         }
       }
+      if constexpr (VEC) ps_cur = ps_nxt;
       fwht_regs<kChunk>(y, h);
+      auto lane_stage = [&](auto jt) {
+        constexpr int J = decltype(jt)::value;
+        if (J * kChunk < h) {
+          // upper lane of a pair: other - y = other + (-y); lower lane: y + other
+          const uint32_t neg = (lane & J) ? 0x80000000u : 0u;
 #pragma unroll
-      for (int j = 1; j < 64; j <<= 1) {
-        if (j * kChunk < h) {
-          const bool upper = (lane & j) != 0;
-#pragma unroll
-          for (int e = 0; e < kChunk; ++e) {
-            const float other = __shfl_xor(y[e], j, 64);
-            y[e] = upper ? other - y[e] : y[e] + other;
-          }
+          for (int e = 0; e < kChunk; ++e) y[e] = lane_xor<J>(y[e]) + __uint_as_float(__float_as_uint(y[e]) ^ neg);
         }
-      }
+      };
+      lane_stage(std::integral_constant<int, 1>{});
+      lane_stage(std::integral_constant<int, 2>{});
+      lane_stage(std::integral_constant<int, 4>{});
+      lane_stage(std::integral_constant<int, 8>{});
+      lane_stage(std::integral_constant<int, 16>{});
+      lane_stage(std::integral_constant<int, 32>{});
       if constexpr (!BIG) {
         int code[kChunk];
 #pragma unroll
@@ -261,7 +389,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
     __syncthreads();
     constexpr int G = 1 << LOG_G;  // block / 512
     const int groups = static_cast<int>(K >> LOG_G);
-    for (int gi = t; gi < groups; gi += kThreads) {
+    for (int gi = t; gi < groups; gi += nthreads) {
       const int base = (gi >> 9) * h + (gi & (kLaneSpan - 1));
       float z[G];
 #pragma unroll
@@ -286,7 +414,9 @@ template <int DT, bool VEC>
 int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {
   int log_g = 0;
   for (int g = a.block / kLaneSpan; g > 1; g >>= 1) ++log_g;
-  dim3 grid(static_cast<unsigned>(a.M)), block(kThreads);
+  // a wavefront owns 512 consecutive elements of a pass: launch only the wavefronts a single-pass row needs
+  const int waves = a.K >= 3 * kLaneSpan ? 4 : static_cast<int>((a.K + kLaneSpan - 1) / kLaneSpan);
+  dim3 grid(static_cast<unsigned>(a.M)), block(64 * waves);
 #define OQ_RQ_CASE(LG)                                                                           \
   case LG: {                                                                                     \
     auto kern = rotate_quantize_kernel<DT, VEC, LG>;                                             \
@@ -358,12 +488,13 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
 
   const size_t kp = static_cast<size_t>(a.passes) * kPass;
   const bool big = block > kLaneSpan;
-  const size_t smem = kp * sizeof(float) + (256 + 256 + 4) * sizeof(float) + (big ? kp : 0);
 
   auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   const bool vec = (K % 8 == 0) && aligned16(x) && aligned16(perm) && aligned16(signs) &&
                    (codes_out == nullptr || aligned16(codes_out)) &&
                    (values_out == nullptr || aligned16(values_out));
+  const bool stage16 = vec && x_dtype != OQ_F32 && !big;  // RqStage::k16
+  const size_t smem = (256 + 256 + 4) * sizeof(float) + kp * (stage16 ? 2 : 4) + (big ? kp : 0);
   switch (x_dtype) {
     case OQ_F32: return vec ? launch_for_block<OQ_F32, true>(a, smem, stream) : launch_for_block<OQ_F32, false>(a, smem, stream);
     case OQ_F16: return vec ? launch_for_block<OQ_F16, true>(a, smem, stream) : launch_for_block<OQ_F16, false>(a, smem, stream);

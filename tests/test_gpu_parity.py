@@ -266,6 +266,21 @@ def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
     check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, f"tile {tile}")
 
 
+@pytest.mark.parametrize(("m", "n", "k", "wbits"), [(300, 200, 1024, 4), (128, 96, 256, 4), (515, 1152, 2304, 3), (130, 104, 512, 6)])
+def test_packed_linear_k_split_kernel(dev, m, n, k, wbits, monkeypatch):
+    """Four wavefronts share one output tile and a quarter of K each; partial tiles are summed through LDS."""
+    monkeypatch.setenv("OQ_GEMM_TILE", "4")
+    rng = np.random.default_rng(m + n + k)
+    layer = make_layer(rng, n, k, wbits, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    got = run_packed_linear(dev, layer, codes, s, "nibble")
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "k-split")
+    again = run_packed_linear(dev, layer, codes, s, "nibble")
+    assert torch.equal(got, again)  # fixed summation order: bitwise reproducible
+
+
 @pytest.mark.parametrize("m", [1, 4, 16, 3])
 @pytest.mark.parametrize(("n", "k", "wbits"), [(4096, 4096, 2), (1000, 4096, 3), (4096, 14336, 3), (2048, 4096, 4), (512, 1152, 6), (256, 1024, 8)])
 def test_packed_linear_small_m_stream_kernel(dev, m, n, k, wbits):
