@@ -35,6 +35,7 @@ def parse_args():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--m", type=int, default=0, help="token count override (c5: 1, 4 or 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
     ap.add_argument("--kernel-iters", type=int, default=50)
     return ap.parse_args()
 
@@ -120,6 +121,49 @@ def run_step(layers, x):
         elif act == "slice3072":
             h = h[..., :3072].contiguous()
     return h
+
+
+# ------------------------------------------------------------------ graph replay
+
+def capture_step(fn, replays_checked=3):
+    """Capture one step into a HIP graph and check every one of a few replays against the eager
+    result (with eager work and synchronisation between replays).  Returns (replay, out) or None
+    when capture is unavailable or a replay differs."""
+    try:
+        ref = fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = fn()
+        for _ in range(replays_checked):
+            graph.replay()
+            torch.cuda.synchronize()
+            again = fn()          # eager work between replays
+            torch.cuda.synchronize()
+            if not (torch.equal(out, ref) and torch.equal(again, ref)):
+                return None
+        return graph.replay, out
+    except Exception as exc:  # capture not supported here: fall back to eager timing
+        print(f"bench.py: graph capture unavailable ({exc}); timing eager launches", file=sys.stderr)
+        return None
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
 
 
 # ------------------------------------------------------------ kernel-only timing
@@ -337,14 +381,17 @@ def bench_c5(args, device):
         for l in mats:
             l(x4096 if l.in_features == 4096 else x14336)
 
-    for _ in range(args.warmup):
-        full_step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        full_step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    def full_step_out():
+        last = None
+        for l in mats:
+            last = l(x4096 if l.in_features == 4096 else x14336)
+        return last
+
+    eager_dt = time_steps(full_step, args.steps, args.warmup)
+    dt, launch = eager_dt, "eager"
+    captured = None if args.no_graph else capture_step(full_step_out)
+    if captured is not None:
+        dt, launch = time_steps(captured[0], args.steps, args.warmup), "hipgraph"
 
     # kernel-only: every matmul launch of the stack, events on the launch stream
     per_stack = time_kernel(stack_matmuls, max(3, args.kernel_iters // 10))
@@ -364,7 +411,8 @@ def bench_c5(args, device):
         "value": packed_bytes / dt / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "config": {"workload": f"c5 40-layer decode stack W2/W3/W4 A4, M={m}", "M": m,
-                                        "packed_bytes_per_step": packed_bytes},
+                                        "packed_bytes_per_step": packed_bytes, "launch": launch,
+                                        "eager_ms_per_step": eager_dt * 1e3},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("c5_gemv_w4_4096x14336"),
                      "kernel": "packed_gemv_kernel<4> on 4096->14336 W4", "bytes_per_launch": w4_bytes,
@@ -398,14 +446,11 @@ def main() -> int:
     x = make_input(spec, spec["layers"][0][0], gen).to(device)
     flops = sum(2.0 * spec["M"] * n * k for (k, n, *_rest) in spec["layers"])
 
-    for _ in range(args.warmup):
-        run_step(layers, x)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step(layers, x)
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    eager_dt = time_steps(lambda: run_step(layers, x), args.steps, args.warmup)
+    dt, launch = eager_dt, "eager"
+    captured = None if args.no_graph else capture_step(lambda: run_step(layers, x))
+    if captured is not None:
+        dt, launch = time_steps(captured[0], args.steps, args.warmup), "hipgraph"
 
     # dominant kernel alone: the packed GEMM of the first layer, and every other piece for the record
     pieces = {}
@@ -430,7 +475,7 @@ def main() -> int:
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": spec["name"], "M": spec["M"], "input_dtype": str(spec["dtype"]).replace("torch.", ""),
-                   "flop_per_step": flops},
+                   "flop_per_step": flops, "launch": launch, "eager_ms_per_step": eager_dt * 1e3},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded_traffic(f"{args.workload}_gemm"),
                      "kernel": "packed_gemm_kernel", "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},

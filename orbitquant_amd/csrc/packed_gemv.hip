@@ -102,9 +102,9 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     }
   };
 
-  // Order of the global loads matters: loads of one wavefront return in order, so the few
-  // centroid values the table build needs go first, then both batches of packed data; the
-  // tables are written while the packed data is still in flight.
+  // The lookup tables are built before the packed stream is requested: the few centroid loads
+  // they need would otherwise queue behind the bulk loads of every workgroup on the CU, and
+  // nothing could be decoded until they came back.
   constexpr int kWEntries = WLut<BITS, kLR>::kEntries;
   const int e_w = tid, e_a = tid - (64 * WAVES - 256);  // last 256 threads build the activation table
   float wv0 = 0.0f, wv1 = 0.0f, av0 = 0.0f, av1 = 0.0f;
@@ -133,8 +133,6 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     }
   }
   Batch b0, b1;
-  if (s_begin < s_end) fetch(s_begin, b0);
-  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
   if (e_w < kWEntries) {
     const uint32_t d = pack16(wv0, wv1, false);
     uint4 *dst = reinterpret_cast<uint4 *>(wlut + (e_w << kLR));
@@ -148,6 +146,8 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     for (int i = 0; i < (1 << kLR) / 4; ++i) dst[i] = make_uint4(d, d, d, d);
   }
   __syncthreads();
+  if (s_begin < s_end) fetch(s_begin, b0);
+  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
 
   for (int s = s_begin; s < s_end; s += 2 * kDepth) {
     consume(s, b0);
