@@ -12,6 +12,14 @@
 // K is cut like in the tiled GEMM: in a K-step of 128, lane group g (0..3) owns
 // the contiguous run k0+32g .. k0+32g+31 of its row and MFMA q (0..3) consumes
 // values 8q..8q+7 of every run.
+//
+// Lookup tables: the 64 KB block of 256-byte rows the tiled GEMM uses (weight
+// entry e 32 times in bytes 0..127 of row e, activation entry e in bytes
+// 128..255; lane l reads copy l%32, a byte-indexed lookup is one v_perm_b32 plus
+// one ds_read_b32).  The packed stream is requested first thing; the tables are
+// built meanwhile from centroids fetched with SCALAR loads, which do not queue
+// behind the vector loads of the stream, and spread over the lanes so that every lane can pick the two values of its table entry with
+// wavefront shuffles.  After the main loop the same LDS holds the partial sums.
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -36,20 +44,40 @@ struct GemvArgs {
   int out_dtype;
 };
 
-constexpr int kLR = 3;     // 8 copies per table entry
-constexpr int kDepth = 2;  // K-steps of 128 fetched per batch of global loads (two batches in flight)
+constexpr int kDepth = 1;  // K-steps of 128 fetched per batch of global loads (two batches in flight: decode of one overlaps the stream of the next)
+constexpr int kGemvTableBytes = 65536;
+
+__device__ __forceinline__ uint32_t gemv_row_address(uint32_t word, uint32_t lane_off, int p) {
+  return __builtin_amdgcn_perm(word, lane_off, 0x03020400u + (static_cast<uint32_t>(p) << 8));
+}
+__device__ __forceinline__ uint4 gemv_decode_bytes(uint32_t f, uint32_t lane_off) {
+  return make_uint4(lds_read_u32(gemv_row_address(f, lane_off, 0)), lds_read_u32(gemv_row_address(f, lane_off, 1)),
+                    lds_read_u32(gemv_row_address(f, lane_off, 2)), lds_read_u32(gemv_row_address(f, lane_off, 3)));
+}
+
+// centroid i (i < COUNT <= 64) into lane i of one register, from scalar loads
+template <int COUNT>
+__device__ __forceinline__ float lane_table(const float *__restrict__ cents, int valid) {
+  const int lane = threadIdx.x & 63;
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i) {
+    const float c = i < valid ? cents[i] : 0.0f;  // uniform address: a scalar load
+    t = lane == i ? c : t;
+  }
+  return t;
+}
 
 template <int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
-  extern __shared__ __align__(16) uint32_t lds[];
-  uint32_t *wlut = lds;
-  uint32_t *alut = lds + WLut<BITS, kLR>::kDwords;
-  float *partial = reinterpret_cast<float *>(alut + alut_dwords<kLR>());  // [WAVES][R][64][4]
+  static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
+  __shared__ __attribute__((aligned(65536))) uint32_t lds[kGemvTableBytes / 4];
+  float *partial = reinterpret_cast<float *>(lds);  // [WAVES][R][64][4], after the main loop
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, grp = lane >> 4;
-  const uint32_t wbase = lds_byte_address(wlut) + 4 * (lane & ((1 << kLR) - 1));
-  const uint32_t abase = lds_byte_address(alut) + 4 * (lane & ((1 << kLR) - 1));
+  const uint32_t lds_base = lds_byte_address(lds);  // a multiple of 65536 by the alignment
+  const uint32_t w_off = lds_base + 4 * (lane & 31), a_off = lds_base + 128 + 4 * (lane & 31);
   const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * R);
 
   const int steps = static_cast<int>(g.K / 128);
@@ -90,10 +118,12 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint32_t f = q == 0 ? bt.a[d].x : q == 1 ? bt.a[d].y : q == 2 ? bt.a[d].z : bt.a[d].w;
-          const uint4 af = decode_a_nibble<kLR>(f, abase);
+          const uint4 af = gemv_decode_bytes(f, a_off);
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-            const uint4 bf = decode_w<BITS, kLR>(bt.w[d][j], q, wbase);
+            uint4 bf;
+            if constexpr (BITS == 4) bf = gemv_decode_bytes(bt.w[d][j][q], w_off);
+            else bf = decode_w<BITS, 6>(bt.w[d][j], q, w_off);
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
                                                              __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
           }
@@ -102,23 +132,11 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     }
   };
 
-  // The lookup tables are built before the packed stream is requested: the few centroid loads
-  // they need would otherwise queue behind the bulk loads of every workgroup on the CU, and
-  // nothing could be decoded until they came back.
-  constexpr int kWEntries = WLut<BITS, kLR>::kEntries;
-  const int e_w = tid, e_a = tid - (64 * WAVES - 256);  // last 256 threads build the activation table
-  float wv0 = 0.0f, wv1 = 0.0f, av0 = 0.0f, av1 = 0.0f;
-  if (e_w < kWEntries) {
-    const int c0 = WLut<BITS>::kPair ? (e_w & ((1 << BITS) - 1)) : e_w;
-    const int c1 = WLut<BITS>::kPair ? (e_w >> BITS) : e_w;
-    wv0 = g.w_cents[c0];
-    wv1 = g.w_cents[c1];
-  }
-  if (e_a >= 0) {
-    const int c0 = e_a & 15, c1 = e_a >> 4;
-    av0 = c0 < g.a_levels ? g.act_cents[c0] : 0.0f;
-    av1 = c1 < g.a_levels ? g.act_cents[c1] : 0.0f;
-  }
+  // ---- the packed stream first ------------------------------------------------------
+  Batch b0, b1;
+  if (s_begin < s_end) fetch(s_begin, b0);
+  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
+
   // epilogue operands of the item this thread will finish (item = tid when tid < 64*R)
   const int ep_j = tid >> 6, ep_l = tid & 63;
   const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
@@ -132,22 +150,37 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
       if (g.row_scale != nullptr && m < g.M) ep_sc[e] = g.row_scale[m];
     }
   }
-  Batch b0, b1;
-  if (e_w < kWEntries) {
-    const uint32_t d = pack16(wv0, wv1, false);
-    uint4 *dst = reinterpret_cast<uint4 *>(wlut + (e_w << kLR));
+
+  // ---- tables: wavefront w writes rows [w*256/WAVES, (w+1)*256/WAVES) ------------------------
+  {
+    constexpr int kLevels = 1 << BITS;
+    constexpr bool kPair = BITS <= 4;
+    constexpr int kRowsPerWave = 256 / WAVES;          // 64, 32 or 16
+    constexpr int kRowsPerWrite = 4;                    // 64 lanes x 16 bytes = four 256-byte rows
+    const float a_tab = lane_table<16>(g.act_cents, g.a_levels);
+    float w_tab = 0.0f;
+    if constexpr (kLevels <= 64) w_tab = lane_table<kLevels>(g.w_cents, kLevels);
 #pragma unroll
-    for (int i = 0; i < (1 << kLR) / 4; ++i) dst[i] = make_uint4(d, d, d, d);
-  }
-  if (e_a >= 0) {
-    const uint32_t d = pack16(av0, av1, false);
-    uint4 *dst = reinterpret_cast<uint4 *>(alut + (e_a << kLR));
-#pragma unroll
-    for (int i = 0; i < (1 << kLR) / 4; ++i) dst[i] = make_uint4(d, d, d, d);
+    for (int i = 0; i < kRowsPerWave / kRowsPerWrite; ++i) {
+      const int e = wave * kRowsPerWave + kRowsPerWrite * i + (lane >> 4);  // the row this lane writes to
+      const uint32_t ea = pack16(__shfl(a_tab, e & 15), __shfl(a_tab, e >> 4), false);
+      uint32_t ew;
+      if constexpr (kLevels <= 64) {
+        if constexpr (kPair) {
+          ew = (e < kLevels * kLevels) ? pack16(__shfl(w_tab, e & (kLevels - 1)), __shfl(w_tab, (e >> BITS) & (kLevels - 1)), false) : 0u;
+        } else {
+          const float v = __shfl(w_tab, e & (kLevels - 1));
+          ew = (e < kLevels) ? pack16(v, v, false) : 0u;
+        }
+      } else {
+        const float v = g.w_cents[e];  // 256 single-code entries: one vector load per row
+        ew = pack16(v, v, false);
+      }
+      const uint32_t d = (lane & 8) ? ea : ew;
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + e * 256 + (lane & 15) * 16) = make_uint4(d, d, d, d);
+    }
   }
   __syncthreads();
-  if (s_begin < s_end) fetch(s_begin, b0);
-  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
 
   for (int s = s_begin; s < s_end; s += 2 * kDepth) {
     consume(s, b0);
@@ -156,7 +189,8 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     if (s + 3 * kDepth < s_end) fetch(s + 3 * kDepth, b1);
   }
 
-  // ---- cross-wave sum in LDS, fixed order ----------------------------------------
+  // ---- cross-wave sum in LDS (the tables are dead), fixed order ------------------------
+  __syncthreads();
 #pragma unroll
   for (int j = 0; j < R; ++j)
     *reinterpret_cast<float4 *>(partial + ((wave * R + j) * 64 + lane) * 4) =
@@ -187,14 +221,8 @@ template <int BITS, int R, int WAVES>
 int launch(const GemvArgs &g, hipStream_t stream) {
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
   if (groups > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: N too large");
-  const size_t smem = (WLut<BITS, kLR>::kDwords + alut_dwords<kLR>()) * sizeof(uint32_t) + sizeof(float) * WAVES * R * 64 * 4;
   auto kern = packed_gemv_kernel<BITS, R, WAVES>;
-  if (smem > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(smem)) != hipSuccess)
-      return fail(OQ_ERR_LAUNCH, "packed_gemv: cannot reserve %zu bytes of LDS", smem);
-  }
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), smem, stream, g);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), 0, stream, g);
   return check_launch("packed_gemv");
 }
 
