@@ -169,14 +169,37 @@ def time_steps(fn, steps, warmup):
 # ------------------------------------------------------------ kernel-only timing
 
 def time_kernel(fn, iters):
+    """Average device time of one call of `fn` (one kernel launch), events on the launch stream.
+    The `iters` launches are replayed from a HIP graph when capture works, so that the figure is
+    the kernel's and not the Python wrapper's (a short kernel is otherwise host-bound)."""
     for _ in range(5):
         fn()
     torch.cuda.synchronize()
+    replay = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(iters):
+                fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        replay = graph.replay
+    except Exception:
+        replay = None
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
     start.record()
-    for _ in range(iters):
-        fn()
+    if replay is not None:
+        replay()
+    else:
+        for _ in range(iters):
+            fn()
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / iters * 1e-3  # seconds per launch
