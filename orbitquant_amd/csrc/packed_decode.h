@@ -129,6 +129,106 @@ __device__ __forceinline__ uint4 decode_a_nibble(uint32_t f, uint32_t base) {
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+
+// ---- the 64 KB table block shared by the tiled GEMM and the small-M kernel -------------------
+// 256 rows of 256 bytes at a 65536-aligned LDS address.  Row e holds, 32 times each, the dword
+// of weight-table entry e (bytes 0..127) and of activation-table entry e (bytes 128..255); lane l
+// reads copy l%32, so the lanes of a wavefront never collide on a bank whatever codes they hold.
+// The activation table and the 4-bit weight table are indexed by a whole byte of the packed
+// stream (two codes) and return both bf16 values in one dword; because a row is 256 bytes the
+// LDS address of such a lookup is "byte 0 = the lane's offset, byte 1 = the code byte", which one
+// v_perm_b32 assembles.  Other weight widths index the same rows with a bit-field extract (pair
+// tables for 2/3 bits, single-code tables for 6/8).
+constexpr int kRowTableBytes = 65536;
+
+__device__ __forceinline__ uint32_t row_address(uint32_t word, uint32_t lane_off, int p) {
+  return __builtin_amdgcn_perm(word, lane_off, 0x03020400u + (static_cast<uint32_t>(p) << 8));
+}
+
+__device__ __forceinline__ uint4 decode_bytes(uint32_t f, uint32_t lane_off) {
+  return make_uint4(lds_read_u32(row_address(f, lane_off, 0)), lds_read_u32(row_address(f, lane_off, 1)),
+                    lds_read_u32(row_address(f, lane_off, 2)), lds_read_u32(row_address(f, lane_off, 3)));
+}
+
+// centroid i (i < COUNT <= 64) into lane i of one register.  The addresses are uniform, so the
+// values come through scalar loads, which do not queue behind the wavefront's vector loads.
+template <int COUNT>
+__device__ __forceinline__ float lane_table(const float *__restrict__ cents, int valid) {
+  const int lane = threadIdx.x & 63;
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i) {
+    const float c = i < valid ? cents[i] : 0.0f;
+    t = lane == i ? c : t;
+  }
+  return t;
+}
+
+// Build the block with WAVES wavefronts: wavefront w writes rows [w*256/WAVES, (w+1)*256/WAVES),
+// four rows per 16-byte-per-lane store.  The caller puts a barrier between this and the first lookup.
+template <int BITS, int WAVES>
+__device__ __forceinline__ void build_row_tables(uint32_t *lds, const float *__restrict__ w_cents,
+                                                 const float *__restrict__ act_cents, int a_levels) {
+  constexpr int kLevels = 1 << BITS;
+  constexpr bool kPair = BITS <= 4;
+  constexpr int kRowsPerWave = 256 / WAVES;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float a_tab = lane_table<16>(act_cents, a_levels);
+  float w_tab = 0.0f;
+  if constexpr (kLevels <= 64) w_tab = lane_table<kLevels>(w_cents, kLevels);
+#pragma unroll
+  for (int i = 0; i < kRowsPerWave / 4; ++i) {
+    const int e = wave * kRowsPerWave + 4 * i + (lane >> 4);  // the row this lane writes to
+    const uint32_t ea = pack16(__shfl(a_tab, e & 15), __shfl(a_tab, e >> 4), false);
+    uint32_t ew;
+    if constexpr (kLevels <= 64) {
+      if constexpr (kPair) {
+        ew = (e < kLevels * kLevels)
+                 ? pack16(__shfl(w_tab, e & (kLevels - 1)), __shfl(w_tab, (e >> BITS) & (kLevels - 1)), false)
+                 : 0u;
+      } else {
+        const float v = __shfl(w_tab, e & (kLevels - 1));
+        ew = (e < kLevels) ? pack16(v, v, false) : 0u;
+      }
+    } else {
+      const float v = w_cents[e];  // 256 single-code entries: one vector load per row
+      ew = pack16(v, v, false);
+    }
+    const uint32_t d = (lane & 8) ? ea : ew;
+    *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + e * 256 + (lane & 15) * 16) = make_uint4(d, d, d, d);
+  }
+}
+
+// The same block for a 256-thread workgroup whose thread t already holds the two dwords of row t
+// (loaded with its first vector loads, before any bulk load): wavefront w writes rows 64w..64w+63;
+// 16-byte chunk c of a row is a weight copy (c < 8) or an activation copy; lane l writes chunk l%16
+// of row 64w + 4i + l/16.  Fewer shuffles than build_row_tables, at the price of a vector-load latency.
+__device__ __forceinline__ void write_row_tables(uint32_t *lds, uint32_t my_w, uint32_t my_a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int src = 4 * i + (lane >> 4);
+    const uint32_t ew = __shfl(my_w, src), ea = __shfl(my_a, src);
+    const uint32_t d = (lane & 8) ? ea : ew;
+    *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + (64 * wave + src) * 256 + (lane & 15) * 16) =
+        make_uint4(d, d, d, d);
+  }
+}
+
+// dword of weight-table row e
+template <int BITS>
+__device__ __forceinline__ uint32_t w_table_entry(const float *cents, int e) {
+  constexpr int levels = 1 << BITS;
+  if constexpr (BITS <= 4) {
+    if (e >= levels * levels) return 0u;
+    return pack16(cents[e & (levels - 1)], cents[e >> BITS], false);
+  } else {
+    if (e >= levels) return 0u;
+    const float v = cents[e];
+    return pack16(v, v, false);
+  }
+}
+
 template <int BITS>
 __device__ __forceinline__ void load_w(const uint8_t *p, uint32_t (&w)[BITS]) {
   if constexpr (BITS == 4) {

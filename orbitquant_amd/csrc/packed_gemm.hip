@@ -56,32 +56,8 @@ struct GemmArgs {
   int tiles_m, tiles_n;
 };
 
-constexpr int kTableBytes = 65536;
+constexpr int kTableBytes = kRowTableBytes;
 static_assert(kEpiLdsBytes <= kTableBytes, "the epilogue reuses the table block");
-
-// dword of weight-table row e
-template <int BITS>
-__device__ __forceinline__ uint32_t w_table_entry(const float *cents, int e) {
-  constexpr int levels = 1 << BITS;
-  if constexpr (BITS <= 4) {
-    if (e >= levels * levels) return 0u;
-    return pack16(cents[e & (levels - 1)], cents[e >> BITS], false);
-  } else {
-    if (e >= levels) return 0u;
-    const float v = cents[e];
-    return pack16(v, v, false);
-  }
-}
-
-// LDS address of the row selected by byte `p` of `word`: (byte << 8) | lane offset
-__device__ __forceinline__ uint32_t row_address(uint32_t word, uint32_t lane_off, int p) {
-  return __builtin_amdgcn_perm(word, lane_off, 0x03020400u + (static_cast<uint32_t>(p) << 8));
-}
-
-__device__ __forceinline__ uint4 decode_bytes(uint32_t f, uint32_t lane_off) {
-  return make_uint4(lds_read_u32(row_address(f, lane_off, 0)), lds_read_u32(row_address(f, lane_off, 1)),
-                    lds_read_u32(row_address(f, lane_off, 2)), lds_read_u32(row_address(f, lane_off, 3)));
-}
 
 // Workgroup = 4 wavefronts; each wavefront owns FM x FN MFMA tiles of 32x32.
 //   KSPLIT = 1: the wavefronts sit 2x2 on a [64 FM x 64 FN] output tile, each runs over all of K.
@@ -165,17 +141,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   fetch(std::integral_constant<int, 0>{}, 0);
   if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
 
-  {  // tables: wavefront w writes rows 64w..64w+63, 16-byte chunk c of a row is a weight copy
-     // (c < 8) or an activation copy; lane l writes chunk l%16 of row 64w + 4i + l/16
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int src = 4 * i + (lane >> 4);
-      const uint32_t ew = __shfl(my_w, src), ea = __shfl(my_a, src);
-      const uint32_t d = (lane & 8) ? ea : ew;
-      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + (64 * wave + src) * 256 + (lane & 15) * 16) =
-          make_uint4(d, d, d, d);
-    }
-  }
+  write_row_tables(lds, my_w, my_a);
 
   f32x16 acc[FM][FN];
 #pragma unroll

@@ -45,28 +45,7 @@ struct GemvArgs {
 };
 
 constexpr int kDepth = 1;  // K-steps of 128 fetched per batch of global loads (two batches in flight: decode of one overlaps the stream of the next)
-constexpr int kGemvTableBytes = 65536;
-
-__device__ __forceinline__ uint32_t gemv_row_address(uint32_t word, uint32_t lane_off, int p) {
-  return __builtin_amdgcn_perm(word, lane_off, 0x03020400u + (static_cast<uint32_t>(p) << 8));
-}
-__device__ __forceinline__ uint4 gemv_decode_bytes(uint32_t f, uint32_t lane_off) {
-  return make_uint4(lds_read_u32(gemv_row_address(f, lane_off, 0)), lds_read_u32(gemv_row_address(f, lane_off, 1)),
-                    lds_read_u32(gemv_row_address(f, lane_off, 2)), lds_read_u32(gemv_row_address(f, lane_off, 3)));
-}
-
-// centroid i (i < COUNT <= 64) into lane i of one register, from scalar loads
-template <int COUNT>
-__device__ __forceinline__ float lane_table(const float *__restrict__ cents, int valid) {
-  const int lane = threadIdx.x & 63;
-  float t = 0.0f;
-#pragma unroll
-  for (int i = 0; i < COUNT; ++i) {
-    const float c = i < valid ? cents[i] : 0.0f;  // uniform address: a scalar load
-    t = lane == i ? c : t;
-  }
-  return t;
-}
+constexpr int kGemvTableBytes = kRowTableBytes;
 
 template <int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
@@ -118,11 +97,11 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint32_t f = q == 0 ? bt.a[d].x : q == 1 ? bt.a[d].y : q == 2 ? bt.a[d].z : bt.a[d].w;
-          const uint4 af = gemv_decode_bytes(f, a_off);
+          const uint4 af = decode_bytes(f, a_off);
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             uint4 bf;
-            if constexpr (BITS == 4) bf = gemv_decode_bytes(bt.w[d][j][q], w_off);
+            if constexpr (BITS == 4) bf = decode_bytes(bt.w[d][j][q], w_off);
             else bf = decode_w<BITS, 6>(bt.w[d][j], q, w_off);
             acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
                                                              __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
@@ -151,35 +130,8 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
     }
   }
 
-  // ---- tables: wavefront w writes rows [w*256/WAVES, (w+1)*256/WAVES) ------------------------
-  {
-    constexpr int kLevels = 1 << BITS;
-    constexpr bool kPair = BITS <= 4;
-    constexpr int kRowsPerWave = 256 / WAVES;          // 64, 32 or 16
-    constexpr int kRowsPerWrite = 4;                    // 64 lanes x 16 bytes = four 256-byte rows
-    const float a_tab = lane_table<16>(g.act_cents, g.a_levels);
-    float w_tab = 0.0f;
-    if constexpr (kLevels <= 64) w_tab = lane_table<kLevels>(g.w_cents, kLevels);
-#pragma unroll
-    for (int i = 0; i < kRowsPerWave / kRowsPerWrite; ++i) {
-      const int e = wave * kRowsPerWave + kRowsPerWrite * i + (lane >> 4);  // the row this lane writes to
-      const uint32_t ea = pack16(__shfl(a_tab, e & 15), __shfl(a_tab, e >> 4), false);
-      uint32_t ew;
-      if constexpr (kLevels <= 64) {
-        if constexpr (kPair) {
-          ew = (e < kLevels * kLevels) ? pack16(__shfl(w_tab, e & (kLevels - 1)), __shfl(w_tab, (e >> BITS) & (kLevels - 1)), false) : 0u;
-        } else {
-          const float v = __shfl(w_tab, e & (kLevels - 1));
-          ew = (e < kLevels) ? pack16(v, v, false) : 0u;
-        }
-      } else {
-        const float v = g.w_cents[e];  // 256 single-code entries: one vector load per row
-        ew = pack16(v, v, false);
-      }
-      const uint32_t d = (lane & 8) ? ea : ew;
-      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + e * 256 + (lane & 15) * 16) = make_uint4(d, d, d, d);
-    }
-  }
+  // ---- tables (built while the stream is in flight) ---------------------------------------
+  build_row_tables<BITS, WAVES>(lds, g.w_cents, g.act_cents, g.a_levels);
   __syncthreads();
 
   for (int s = s_begin; s < s_end; s += 2 * kDepth) {
