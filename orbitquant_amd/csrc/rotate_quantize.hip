@@ -91,6 +91,28 @@ __device__ __forceinline__ int bucketize(const float *bnd, int levels_pow2, floa
   return code;
 }
 
+// Faster bucketize for small codebooks: the interval [first boundary, last boundary] is cut
+// into kCells(levels) uniform cells; cell c stores how many boundaries lie in lower cells and
+// the one boundary inside it (+inf if none), so a value costs one LDS read and one compare:
+//   code = table[cell(v)].below + (table[cell(v)].boundary < v)
+// This is exact for ANY monotone cell(): boundaries in lower cells are < v, boundaries in
+// higher cells are > v, and the one in v's own cell is compared directly.  The table is only
+// used when no cell holds two boundaries (checked while it is built); otherwise, and for
+// codebooks of more than 64 levels, the binary search above is used.
+constexpr int kMaxCells = 512;
+struct CellMap {
+  float scale, offset;
+  int cells;  // 0: table not usable
+};
+__device__ __forceinline__ int cell_of(const CellMap &m, float v) {
+  const int c = __float2int_rd(__builtin_fmaf(v, m.scale, m.offset));
+  return min(max(c, 0), m.cells - 1);
+}
+__device__ __forceinline__ int bucketize_cells(const uint2 *table, const CellMap &m, float v) {
+  const uint2 e = table[cell_of(m, v)];
+  return static_cast<int>(e.y) + (__uint_as_float(e.x) < v ? 1 : 0);
+}
+
 // Emit eight consecutive results (slots c0 .. c0+7 of `row`).
 template <int DT, bool VEC>
 __device__ __forceinline__ void emit8(const RqArgs &a, int64_t row, int64_t c0, const int (&code)[kChunk],
@@ -231,7 +253,9 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   float *bnd = reinterpret_cast<float *>(smem);  // 256 floats
   float *cent = bnd + 256;                       // 256 floats
   float *red = cent + 256;                       // 4 floats
-  float *xbuf = red + 4;                         // Kp elements of Stage::kBytes
+  uint2 *cells = reinterpret_cast<uint2 *>(red + 4);            // kMaxCells x (boundary, count below)
+  int *cells_bad = reinterpret_cast<int *>(cells + kMaxCells);  // 4 ints (one used)
+  float *xbuf = reinterpret_cast<float *>(cells_bad + 4);       // Kp elements of Stage::kBytes
   uint16_t *xbuf16 = reinterpret_cast<uint16_t *>(xbuf);
   uint8_t *cbuf = reinterpret_cast<uint8_t *>(xbuf) + static_cast<size_t>(Kp) * Stage::kBytes;  // Kp bytes, big-block path only
 
@@ -246,6 +270,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
     bnd[i] = (i < a.levels - 1) ? a.bounds[i] : __builtin_inff();
     cent[i] = (a.cents != nullptr && i < a.levels) ? a.cents[i] : 0.0f;
   }
+  if (t == 0) cells_bad[0] = 0;
 
   // ---- phase A: stage the row, sum of squares in the documented order --------
   const int64_t row_base = row * K;
@@ -296,6 +321,34 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   const bool row_plain = !(denom > 1e-30f && denom < 1e30f);  // the reciprocal itself would lose bits
   if (t == 0 && a.norms != nullptr) a.norms[row] = s_norm;
 
+  // ---- bucketize table (the boundaries are in LDS since the barrier above) ----------------
+  CellMap cmap;
+  cmap.cells = a.levels <= 64 && a.levels >= 3 ? 8 * a.levels_pow2 : 0;
+  {
+    const float lo = bnd[0], hi = bnd[a.levels - 2];
+    cmap.scale = static_cast<float>(cmap.cells) / (hi - lo);
+    cmap.offset = -lo * cmap.scale;
+    if (!(hi > lo) || !(cmap.scale < 3.0e38f) || !(__builtin_fabsf(cmap.offset) < 3.0e38f)) cmap.cells = 0;
+  }
+  if (cmap.cells > 0) {
+    const int nb = a.levels - 1;
+    for (int c = t; c < cmap.cells; c += nthreads) {
+      // boundaries are ascending, so their cells are too: first boundary with cell >= c, first with cell > c
+      int first = 0, last = 0;
+      for (int step = a.levels_pow2; step > 0; step >>= 1) {
+        if (first + step <= nb && cell_of(cmap, bnd[first + step - 1]) < c) first += step;
+        if (last + step <= nb && cell_of(cmap, bnd[last + step - 1]) <= c) last += step;
+      }
+      if (last - first > 1) cells_bad[0] = 1;
+      cells[c] = make_uint2(__float_as_uint(last > first ? bnd[first] : __builtin_inff()), static_cast<uint32_t>(first));
+    }
+    __syncthreads();
+    if (cells_bad[0] != 0) cmap.cells = 0;
+  }
+  auto code_of = [&](float v) -> int {
+    return cmap.cells > 0 ? bucketize_cells(cells, cmap, v) : bucketize(bnd, a.levels_pow2, v);
+  };
+
   auto staged = [&](int i) -> float {
     if constexpr (Stage::k16) {
       if constexpr (DT == OQ_BF16) return bf16_bits_to_f32(xbuf16[i]);
@@ -312,7 +365,8 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
 
 #pragma unroll
   for (int p = 0; p < kMaxPasses; ++p) {
-    if (p < a.passes) {
+    // small blocks: a wavefront whose 512 slots of this pass all lie past the row has nothing to do
+    if (p < a.passes && (BIG || static_cast<int64_t>(p) * kPass + (t & ~63) * kChunk < K)) {
       const int64_t c0 = static_cast<int64_t>(p) * kPass + t * kChunk;
       float y[kChunk];
       if constexpr (VEC) {
@@ -366,7 +420,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
       if constexpr (!BIG) {
         int code[kChunk];
 #pragma unroll
-        for (int e = 0; e < kChunk; ++e) code[e] = bucketize(bnd, a.levels_pow2, y[e] * a.inv_sqrt_block);
+        for (int e = 0; e < kChunk; ++e) code[e] = code_of(y[e] * a.inv_sqrt_block);
         if (c0 < K) emit8<DT, VEC>(a, row, c0, code, cent, s_norm);
       } else {
 #pragma unroll
@@ -397,7 +451,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
       fwht_regs<G>(z, G);
 #pragma unroll
       for (int v = 0; v < G; ++v)
-        cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(bucketize(bnd, a.levels_pow2, z[v] * a.inv_sqrt_block));
+        cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(code_of(z[v] * a.inv_sqrt_block));
     }
     __syncthreads();
     for (int64_t c0 = t * kChunk; c0 < K; c0 += kPass) {
@@ -494,7 +548,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                    (codes_out == nullptr || aligned16(codes_out)) &&
                    (values_out == nullptr || aligned16(values_out));
   const bool stage16 = vec && x_dtype != OQ_F32 && !big;  // RqStage::k16
-  const size_t smem = (256 + 256 + 4) * sizeof(float) + kp * (stage16 ? 2 : 4) + (big ? kp : 0);
+  const size_t smem = (256 + 256 + 4) * sizeof(float) + kMaxCells * 8 + 16 + kp * (stage16 ? 2 : 4) + (big ? kp : 0);
   switch (x_dtype) {
     case OQ_F32: return vec ? launch_for_block<OQ_F32, true>(a, smem, stream) : launch_for_block<OQ_F32, false>(a, smem, stream);
     case OQ_F16: return vec ? launch_for_block<OQ_F16, true>(a, smem, stream) : launch_for_block<OQ_F16, false>(a, smem, stream);
