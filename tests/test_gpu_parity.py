@@ -129,6 +129,41 @@ def test_rotate_quantize_one_hot_rows(dev, dim):
     assert np.array_equal(nib.cpu().numpy(), o.pack_nibbles(np.stack(rows)))
 
 
+@pytest.mark.parametrize("kind", ["clustered", "duplicates", "one_sided", "wide_range", "two_levels", "sixty_four"])
+def test_rotate_quantize_awkward_boundaries(dev, kind):
+    """Boundary sets that defeat (or stress) the kernel's uniform cell table: the codes must still be
+    the count of boundaries below each value, ties included."""
+    rng = np.random.default_rng(len(kind))
+    dim, block, rows = 256, 64, 24
+    if kind == "clustered":       # several boundaries closer together than a cell: binary-search fallback
+        bounds = np.array([-0.3, -0.1, -1e-6, 0.0, 1e-7, 2e-7, 3e-7, 0.05, 0.05001, 0.1, 0.11, 0.2, 0.21, 0.3, 0.31], dtype=F32)
+    elif kind == "duplicates":
+        bounds = np.array([-0.2, -0.1, -0.1, 0.0, 0.0, 0.0, 0.1, 0.1, 0.15, 0.2, 0.25, 0.3, 0.3, 0.4, 0.5], dtype=F32)
+    elif kind == "one_sided":
+        bounds = np.linspace(0.01, 0.2, 15, dtype=F32)
+    elif kind == "wide_range":    # every value falls into the first or last cells
+        bounds = np.linspace(-1e6, 1e6, 15, dtype=F32)
+    elif kind == "two_levels":
+        bounds = np.array([0.0], dtype=F32)
+    else:
+        bounds = np.sort(rng.standard_normal(63).astype(F32) * 0.08)
+    perm, signs, block, inv = o.rpbh_constants(dim, 3, block)
+    x32 = rng.standard_normal((rows, dim)).astype(F32)
+    x32[1] = 0
+    # rows that land exactly on boundaries after rotation are rare; force ties through a one-hot row whose
+    # rotated entries are +-inv and boundaries that include those very values
+    x32[2] = 0
+    x32[2, 5] = 1.0
+    if kind == "clustered":
+        bounds[0], bounds[-1] = -inv, inv
+        bounds = np.sort(bounds)
+    xt = torch.from_numpy(x32)
+    want_codes, want_norms = oracle_c.rotate_quantize(x32, perm, signs, bounds, block, 1e-10, inv)
+    codes, _, norms = gpu_rotate_quantize(dev, xt, perm, signs, bounds, block, 1e-10, inv, None, "u8")
+    assert np.array_equal(norms.cpu().numpy().view(np.int32), want_norms.view(np.int32))
+    assert np.array_equal(codes.cpu().numpy(), want_codes)
+
+
 def test_rotate_quantize_full_size_c2_bit_exact(dev):
     # BASELINE config 2, second quantizer: [2048, 4608] bf16 with outlier columns x30
     rng = np.random.default_rng(2)
