@@ -205,22 +205,30 @@ def time_kernel(fn, iters):
     return start.elapsed_time(stop) / iters * 1e-3  # seconds per launch
 
 
+def _code_format(layer, x):
+    """The activation-code format OrbitLinear's forward picks for this input (orbitquant_amd/layers.py)."""
+    if layer.activation_bits <= 4:
+        return "nibble"
+    return "u8" if x.numel() // layer.in_features > 16 and layer.in_features % 64 == 0 else None
+
+
 def gemm_only_closure(layer, x):
     """The matmul launch of `layer` alone, on pre-computed activation codes."""
     from orbitquant_amd import ops
 
     k = layer.in_features
-    if layer.activation_bits <= 4:
+    fmt = _code_format(layer, x)
+    if fmt is not None:
         codes, _, norms = ops.rotate_quantize(
             x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
             block_size=layer.rotation.block_size, eps=layer.activation_eps,
-            inv_sqrt_block=layer.rotation.normalization, code_format="nibble")
+            inv_sqrt_block=layer.rotation.normalization, code_format=fmt)
         bias = layer.bias
 
         def fn():
             return ops.packed_linear(
                 codes, norms, layer._activation_codebook_centroids, layer.packed_weight_indices, layer.row_norms,
-                layer._weight_codebook_centroids, code_format="nibble", activation_bits=layer.activation_bits,
+                layer._weight_codebook_centroids, code_format=fmt, activation_bits=layer.activation_bits,
                 weight_bits=layer.weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
                 output_dtype=x.dtype)
         return fn
@@ -242,7 +250,7 @@ def gemm_only_closure(layer, x):
 def quantize_only_closure(layer, x):
     from orbitquant_amd import ops
 
-    fmt = "nibble" if layer.activation_bits <= 4 else None
+    fmt = _code_format(layer, x)
     vals = None if fmt else "unit_bf16"
 
     def fn():
@@ -483,7 +491,7 @@ def main() -> int:
         tq = time_kernel(quantize_only_closure(layer, h), args.kernel_iters)
         tg = time_kernel(gemm_only_closure(layer, h), args.kernel_iters)
         elem = 4 if h.dtype == torch.float32 else 2
-        q_bytes = spec["M"] * k * elem + spec["M"] * k * (0.5 if layer.activation_bits <= 4 else 2) + 4 * spec["M"]
+        q_bytes = spec["M"] * k * elem + spec["M"] * k * {"nibble": 0.5, "u8": 1, None: 2}[_code_format(layer, h)] + 4 * spec["M"]
         pieces[f"layer{i}"] = {
             "shape": [spec["M"], n, k], "gemm_us": tg * 1e6, "gemm_tflops": 2.0 * spec["M"] * n * k / tg / 1e12,
             "quantize_us": tq * 1e6, "quantize_gbs": q_bytes / tq / 1e9}

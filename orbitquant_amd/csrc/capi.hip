@@ -124,8 +124,8 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
   if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
     return gemv_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
-  if (fast_ptrs && tiled_out && code_format == OQ_CODES_NIBBLE && gemm_supported(K, w_bits))
-    return gemm_dispatch(0, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
+  if (fast_ptrs && tiled_out && gemm_supported(K, w_bits) && (code_format == OQ_CODES_NIBBLE || M > 16))
+    return gemm_dispatch(code_format == OQ_CODES_NIBBLE ? 0 : 1, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
   return generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
                               w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);

@@ -38,10 +38,10 @@
 namespace oq {
 namespace {
 
-enum AMode { A_NIBBLE = 0 };
+enum AMode { A_NIBBLE = 0, A_U8 = 1 };  // activation codes: two per byte, or one per byte
 
 struct GemmArgs {
-  const uint8_t *a;          // [M, K/2] nibble codes
+  const uint8_t *a;          // [M, K/2] nibble codes or [M, K] one code per byte
   const float *row_scale;    // [M] or NULL
   const float *act_cents;    // [a_levels]
   int a_levels;
@@ -79,9 +79,12 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // are written while the packed data is still in flight.
   const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
   uint32_t my_a;
-  {
+  if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
     const int c0 = tid & 15, c1 = tid >> 4;
     my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
+  } else {                         // row = one code, its value in both halves of the dword
+    const float v = tid < g.a_levels ? g.act_cents[tid] : 0.0f;
+    my_a = pack16(v, v, false);
   }
 
   constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
@@ -107,22 +110,24 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   EpiFactors<FM> epi;
   gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
 
-  const int64_t a_row_bytes = g.K / 2;
+  constexpr int kAStep = AM == A_NIBBLE ? 32 : 64;  // bytes of one activation row per K-step of 64
+  constexpr int kAVec = kAStep / 32;                // 16-byte loads per lane per K-step
+  const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K;
   const int64_t w_row_bytes = g.K * BITS / 8;
   const uint8_t *ap[FM];
   const uint8_t *wp[FN];
 #pragma unroll
-  for (int i = 0; i < FM; ++i) ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * 16;
+  for (int i = 0; i < FM; ++i) ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
 #pragma unroll
   for (int j = 0; j < FN; ++j) wp[j] = g.w + min(n_base + 32 * j + r, g.N - 1) * w_row_bytes + grp * (4 * BITS);
 
   // packed operands of NBUF consecutive K-steps
-  uint4 pa[NBUF][FM];
+  uint4 pa[NBUF][FM][kAVec];
   uint32_t pw[NBUF][FN][BITS];
   const int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
   if constexpr (KSPLIT > 1) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * 32;
+    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * kAStep;
 #pragma unroll
     for (int j = 0; j < FN; ++j) wp[j] += static_cast<int64_t>(wave) * steps * (8 * BITS);
   }
@@ -130,7 +135,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   auto fetch_one = [&](auto buf, int e, int ks) {
     constexpr int B = decltype(buf)::value;
     const int64_t s = min(ks, steps - 1);  // past the end: re-read the last step (never multiplied)
-    if (e < FM) pa[B][e] = *reinterpret_cast<const uint4 *>(ap[e] + s * 32);
+    if (e < FM) {
+#pragma unroll
+      for (int v = 0; v < kAVec; ++v) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + 16 * v);
+    }
     else load_w<BITS>(wp[e - FM] + s * (8 * BITS), pw[B][e - FM]);
   };
   auto fetch = [&](auto buf, int ks) {
@@ -159,46 +167,73 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // may be moved across the boundary between two such groups, so the matrix core never
   // waits behind a burst of lookups and the LDS queue never runs dry.  The first phase of a
   // K-step also carries the FM+FN global loads of the K-step NBUF-1 ahead, one per group.
-  constexpr int kLookups = 4 * (FM + FN), kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
+  //
+  // One-code-per-byte activations take two lookups per operand dword (single-code table, the
+  // value in both halves); the two are merged with one v_perm_b32 when the operand is used.
+  constexpr int kRA = AM == A_NIBBLE ? 4 : 8;  // LDS reads per activation tile and phase
+  constexpr int kLookups = kRA * FM + 4 * FN, kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
   constexpr int kLook = (kLookups + kGroups - 1) / kGroups;
-  uint32_t oa[2][FM][4], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
+  uint32_t oa[2][FM][kRA], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
 
-  // lookup t of a phase, in the order the MFMAs of the next phase want their operands:
-  // A tile 0, every weight tile, then A tiles 1..FM-1.  Split in two halves so that the
-  // address of a lookup is computed one group before its LDS read is issued.
+  // dword d (0..7 for bytes, 0..3 for nibbles) of this lane's activation run in buffer B, tile i
+  auto a_word = [&](auto buf, int i, int d) -> uint32_t {
+    constexpr int B = decltype(buf)::value;
+    const uint4 v = pa[B][i][d >> 2];
+    return (d & 3) == 0 ? v.x : (d & 3) == 1 ? v.y : (d & 3) == 2 ? v.z : v.w;
+  };
+  // Lookup t of a phase, in the order the MFMAs of the next phase want their operands:
+  // activation tile 0, every weight tile, then activation tiles 1..FM-1.  Split in two halves
+  // so that the address of a lookup is computed one group before its LDS read is issued.
   auto lookup_address = [&](auto buf, int q, int t) -> uint32_t {
     constexpr int B = decltype(buf)::value;
-    const int p = t & 3, f = t >> 2;
-    if (f == 0 || f > FN) {
-      const int i = f == 0 ? 0 : f - FN;
-      const uint32_t word = q == 0 ? pa[B][i].x : q == 1 ? pa[B][i].y : q == 2 ? pa[B][i].z : pa[B][i].w;
-      return row_address(word, a_off, p);
+    const bool is_a = t < kRA || t >= kRA + 4 * FN;
+    if (is_a) {
+      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
+      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
+      if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
+      else return row_address(a_word(buf, i, 2 * q + (sub >> 2)), a_off, sub & 3);  // byte 8q + sub of the run
     }
-    if constexpr (BITS == 4) return row_address(pw[B][f - 1][q], w_off, p);
+    const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
+    if constexpr (BITS == 4) return row_address(pw[B][j][q], w_off, p);
     else return 0u;
   };
   auto lookup_read = [&](auto buf, int q, int set, int t, uint32_t address) {
     constexpr int B = decltype(buf)::value;
-    const int p = t & 3, f = t >> 2;
-    if (f == 0 || f > FN) {
-      oa[set][f == 0 ? 0 : f - FN][p] = lds_read_u32(address);
+    const bool is_a = t < kRA || t >= kRA + 4 * FN;
+    if (is_a) {
+      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
+      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
+      oa[set][i][sub] = lds_read_u32(address);
     } else {
-      if constexpr (BITS == 4) ob[set][f - 1][p] = lds_read_u32(address);
-      else ob[set][f - 1][p] = decode_w_piece<BITS, 6>(pw[B][f - 1], q, p, w_off);
+      const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
+      if constexpr (BITS == 4) ob[set][j][p] = lds_read_u32(address);
+      else ob[set][j][p] = decode_w_piece<BITS, 6>(pw[B][j], q, p, w_off);
+    }
+  };
+  // the activation operand of tile i out of `set`
+  auto a_operand = [&](int set, int i) -> uint4 {
+    if constexpr (AM == A_NIBBLE) {
+      return make_uint4(oa[set][i][0], oa[set][i][1], oa[set][i][2], oa[set][i][3]);
+    } else {
+      return make_uint4(__builtin_amdgcn_perm(oa[set][i][1], oa[set][i][0], 0x07060100u),
+                        __builtin_amdgcn_perm(oa[set][i][3], oa[set][i][2], 0x07060100u),
+                        __builtin_amdgcn_perm(oa[set][i][5], oa[set][i][4], 0x07060100u),
+                        __builtin_amdgcn_perm(oa[set][i][7], oa[set][i][6], 0x07060100u));
     }
   };
   // lookups of (buf, q) into `set` interleaved with the MFMAs on the other set
   auto phase = [&](auto buf, int q, int set, auto fetch_buf, int fetch_ks, bool with_fetch) {
     uint32_t addr[2][kLook];
+    uint4 av = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
     for (int t = 0; t < kLookups / kGroups; ++t) addr[0][t] = lookup_address(buf, q, t);
 #pragma unroll
     for (int m = 0; m < kGroups; ++m) {
       const int i = m / FN, j = m % FN;
+      if (j == 0) av = a_operand(set ^ 1, i);
       const int lo = m * kLookups / kGroups, hi = (m + 1) * kLookups / kGroups, hi2 = (m + 2) * kLookups / kGroups;
       if (with_fetch && m < FM + FN) fetch_one(fetch_buf, m, fetch_ks);
       const uint4 bw = make_uint4(ob[set ^ 1][j][0], ob[set ^ 1][j][1], ob[set ^ 1][j][2], ob[set ^ 1][j][3]);
-      const uint4 av = make_uint4(oa[set ^ 1][i][0], oa[set ^ 1][i][1], oa[set ^ 1][i][2], oa[set ^ 1][i][3]);
       // weights first: the accumulator tile is the transposed output tile
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, av),
                                                           acc[i][j], 0, 0, 0);
@@ -224,7 +259,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   };
 
 #pragma unroll
-  for (int t = 0; t < 4 * (FM + FN); ++t)
+  for (int t = 0; t < kLookups; ++t)
     lookup_read(std::integral_constant<int, 0>{}, 0, 0, t, lookup_address(std::integral_constant<int, 0>{}, 0, t));
   int ks = 0;
   for (; ks + NBUF <= steps; ks += NBUF) {
@@ -303,7 +338,11 @@ template <int AM, int BITS>
 int launch_bits(const GemmArgs &g, int tile, hipStream_t stream) {
   if (tile == 4) return launch_cfg<AM, BITS, 4, 3, 4>(g, stream);
   if (tile == 3) return launch_cfg<AM, BITS, 4, 3>(g, stream);
-  if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
+  if constexpr (AM == A_NIBBLE) {
+    if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
+  } else {
+    if (tile == 2) return launch_cfg<AM, BITS, 4, 3>(g, stream);  // byte codes need more registers: 256x192 at most
+  }
   if (tile == 1) return launch_cfg<AM, BITS, 2, 4>(g, stream);
   return launch_cfg<AM, BITS, 2, 2>(g, stream);
 }
@@ -372,8 +411,9 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
   const int tile = gemm_choose_tile(M, N, K);
-  if (a_mode != A_NIBBLE) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
-  return launch_mode<A_NIBBLE>(g, bits, tile, stream);
+  if (a_mode == A_NIBBLE) return launch_mode<A_NIBBLE>(g, bits, tile, stream);
+  if (a_mode == A_U8) return launch_mode<A_U8>(g, bits, tile, stream);
+  return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
 }
 
 }  // namespace oq

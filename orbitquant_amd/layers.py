@@ -54,6 +54,16 @@ def quantized_linear_forward(
             codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
             code_format="nibble", activation_bits=activation_bits, weight_bits=weight_bits,
             out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
+    tokens = x.numel() // in_features
+    if tokens > 16 and in_features % 64 == 0:
+        # wider activation codes, many tokens: one code per byte into the all-table tile kernel
+        codes, _, norms = ops.rotate_quantize(
+            x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
+            inv_sqrt_block=inv_sqrt_block, code_format="u8")
+        return ops.packed_linear(
+            codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
+            code_format="u8", activation_bits=activation_bits, weight_bits=weight_bits,
+            out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
     _, unit, norms = ops.rotate_quantize(
         x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
         inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16")

@@ -288,6 +288,25 @@ def test_packed_linear_tile_kernel(dev, m, n, k, wbits, abits, block, with_bias,
     check_outputs(got_u8.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "u8")
 
 
+@pytest.mark.parametrize(("m", "n", "k", "wbits", "abits"), [
+    (300, 200, 1024, 4, 6), (130, 96, 256, 4, 8), (257, 384, 1536, 3, 6), (64, 64, 64, 2, 5), (100, 136, 512, 6, 6),
+    (90, 72, 384, 8, 8), (515, 520, 1152, 4, 4)])
+@pytest.mark.parametrize("tile", ["0", "1", "3"])
+def test_packed_linear_byte_codes_tile_kernel(dev, m, n, k, wbits, abits, tile, monkeypatch):
+    """One activation code per byte (a_bits up to 8) through the all-table tile kernel."""
+    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+    rng = np.random.default_rng(m + 3 * n + k + wbits + abits + int(tile))
+    layer = make_layer(rng, n, k, wbits, abits)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    x32[2] = 0
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    got = run_packed_linear(dev, layer, codes, s, "u8")
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, f"u8 tile {tile}")
+    expect = np.zeros(n) if layer["bias"] is None else torch.from_numpy(layer["bias"]).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(got[2].float().cpu().numpy(), expect)
+
+
 @pytest.mark.parametrize("tile", ["0", "1", "2", "3"])
 def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
     monkeypatch.setenv("OQ_GEMM_TILE", tile)
