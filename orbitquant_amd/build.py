@@ -31,6 +31,7 @@ SOURCES = {
     "rotate_quantize.hip": ["-ffp-contract=off"],
     "packed_generic.hip": [],
     "packed_gemm.hip": [],
+    "packed_gemm_bytes.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
 }

@@ -1,365 +1,11 @@
-// Packed-weight GEMM on the gfx950 matrix cores: 4-bit activation codes x packed weight indices.
-//
-//   out[m,n] = (sum_k c_a[code[m,k]] * c_w[idx[n,k]]) * scale[m] * r_w[n] + bias[n]
-//
-// code is the nibble stream of activation codes, idx the flat little-endian bit
-// stream of 2/3/4/6/8-bit weight indices, both read from HBM as they are stored.
-// Nothing is dequantized to memory: every wavefront loads the packed dwords of
-// its own rows straight into registers, turns them into bf16 MFMA operands
-// through lookup tables held in LDS, and feeds v_mfma_f32_32x32x16_bf16.
-//
-// Operand layout.  One MFMA consumes, per lane, eight k-values of one row
-// (lane l: row l%32, k-group l/32).  A dot product does not care in which order
-// k is visited as long as both operands agree, so a K-step of 64 is cut as
-//   lane group g (0/1) owns k0+32g .. k0+32g+31   (one contiguous run of bits per row)
-//   MFMA q (0..3) of the step uses values 8q..8q+7 of that run
-// which makes every global load of packed data one contiguous 4*bits-byte run
-// per lane (16 bytes for 4-bit), with no cross-lane shuffles and no LDS staging.
-//
-// Lookup tables.  One 64 KB block of LDS, 256 rows of 256 bytes, placed at LDS
-// address 0.  Row e holds, 32 times each, the dword of weight-table entry e
-// (bytes 0..127) and of activation-table entry e (bytes 128..255); lane l reads
-// copy l%32, so the lanes of a wavefront never collide on a bank whatever codes
-// they hold.  The activation table and the 4-bit weight table are indexed by a
-// whole byte of the packed stream (two codes) and return both bf16 values in one
-// dword, and because a row is 256 bytes the LDS address of a lookup is simply
-//   byte 0 = the lane's offset, byte 1 = the code byte
-// which one v_perm_b32 assembles: a lookup is one VALU instruction plus one
-// ds_read_b32 for two operand values.  Other weight widths index the same rows
-// with a bit-field extract (pair tables for 2/3 bits, single-code for 6/8).
-//
-// The instruction stream of a wavefront is what bounds this kernel (per MFMA of
-// 32 cycles it may issue about eight other instructions), hence the tile shapes:
-// a wavefront owning FM x FN tiles of 32x32 issues 4*(FM+FN) lookups per FM*FN MFMAs.
-#include <type_traits>
+// Tile GEMM, two-4-bit-codes-per-byte activations; tile choice and dispatch for both code formats.
+#include <stdlib.h>
 
-#include "gemm_epilogue.h"
+#include "packed_gemm_kernel.h"
 
 namespace oq {
-namespace {
 
-enum AMode { A_NIBBLE = 0, A_U8 = 1 };  // activation codes: two per byte, or one per byte
-
-struct GemmArgs {
-  const uint8_t *a;          // [M, K/2] nibble codes or [M, K] one code per byte
-  const float *row_scale;    // [M] or NULL
-  const float *act_cents;    // [a_levels]
-  int a_levels;
-  const uint8_t *w;          // packed index stream
-  const uint16_t *row_norms; // bf16 [N]
-  const float *w_cents;      // [2^bits]
-  const void *bias;
-  int bias_dtype;
-  int64_t M, N, K;
-  void *out;
-  int out_dtype;
-  int tiles_m, tiles_n;
-};
-
-constexpr int kTableBytes = kRowTableBytes;
-static_assert(kEpiLdsBytes <= kTableBytes, "the epilogue reuses the table block");
-
-// Workgroup = 4 wavefronts; each wavefront owns FM x FN MFMA tiles of 32x32.
-//   KSPLIT = 1: the wavefronts sit 2x2 on a [64 FM x 64 FN] output tile, each runs over all of K.
-//   KSPLIT = 4: all four work on the SAME [32 FM x 32 FN] output tile, each over a quarter of K
-//               (for short-and-wide problems whose output has too few tiles to fill the chip);
-//               the partial tiles are then summed through LDS in a fixed order, each wavefront
-//               ending up with one 32-row slice of the tile, which it scales and stores.  FM = 4.
-// NBUF = K-steps of packed operands held in registers (NBUF-1 of them in flight from memory).
-template <int AM, int BITS, int FM, int FN, int KSPLIT = 1, int NBUF = (FM * FN >= 12 ? 2 : 3)>
-__global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
-  static_assert(KSPLIT == 1 || (KSPLIT == 4 && FM == 4), "K split: four wavefronts, four row slices");
-  __shared__ __attribute__((aligned(65536))) uint32_t lds[kTableBytes / 4];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, grp = lane >> 5;
-
-  // Loads of one wavefront return in order, so the centroid values this thread needs for its
-  // table row are requested first, then the packed operands of the first K-steps; the tables
-  // are written while the packed data is still in flight.
-  const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
-  uint32_t my_a;
-  if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
-    const int c0 = tid & 15, c1 = tid >> 4;
-    my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
-  } else {                         // row = one code, its value in both halves of the dword
-    const float v = tid < g.a_levels ? g.act_cents[tid] : 0.0f;
-    my_a = pack16(v, v, false);
-  }
-
-  constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
-  // tile order: spread consecutive workgroup ids over the 8 XCDs' private L2s in
-  // contiguous chunks, then walk groups of 4 tile-rows column by column
-  int bid = blockIdx.x;
-  const int total = g.tiles_m * g.tiles_n;
-  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
-  constexpr int GROUP_M = 4;
-  const int width = GROUP_M * g.tiles_n;
-  const int group = bid / width;
-  const int first_m = group * GROUP_M;
-  const int gsz = min(g.tiles_m - first_m, GROUP_M);
-  const int pid_m = first_m + (bid % width) % gsz;
-  const int pid_n = (bid % width) / gsz;
-
-  const uint32_t lds_base = lds_byte_address(lds);           // a multiple of 65536 by the alignment
-  const uint32_t w_off = lds_base + 4 * r, a_off = lds_base + 128 + 4 * r;  // the lane's copy inside a table row
-  const int wm = KSPLIT == 1 ? (wave >> 1) * (FM * 32) : 0, wn = KSPLIT == 1 ? (wave & 1) * (FN * 32) : 0;
-  const int64_t m_base = static_cast<int64_t>(pid_m) * TM + wm;
-  const int64_t n_base = static_cast<int64_t>(pid_n) * TN + wn;
-
-  EpiFactors<FM> epi;
-  gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
-
-  constexpr int kAStep = AM == A_NIBBLE ? 32 : 64;  // bytes of one activation row per K-step of 64
-  constexpr int kAVec = kAStep / 32;                // 16-byte loads per lane per K-step
-  const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K;
-  const int64_t w_row_bytes = g.K * BITS / 8;
-  const uint8_t *ap[FM];
-  const uint8_t *wp[FN];
-#pragma unroll
-  for (int i = 0; i < FM; ++i) ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
-#pragma unroll
-  for (int j = 0; j < FN; ++j) wp[j] = g.w + min(n_base + 32 * j + r, g.N - 1) * w_row_bytes + grp * (4 * BITS);
-
-  // packed operands of NBUF consecutive K-steps
-  uint4 pa[NBUF][FM][kAVec];
-  uint32_t pw[NBUF][FN][BITS];
-  const int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
-  if constexpr (KSPLIT > 1) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * kAStep;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) wp[j] += static_cast<int64_t>(wave) * steps * (8 * BITS);
-  }
-  // operand `e` (A row-tile e < FM, else weight column-tile e-FM) of K-step ks into buffer B
-  auto fetch_one = [&](auto buf, int e, int ks) {
-    constexpr int B = decltype(buf)::value;
-    const int64_t s = min(ks, steps - 1);  // past the end: re-read the last step (never multiplied)
-    if (e < FM) {
-#pragma unroll
-      for (int v = 0; v < kAVec; ++v) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + 16 * v);
-    }
-    else load_w<BITS>(wp[e - FM] + s * (8 * BITS), pw[B][e - FM]);
-  };
-  auto fetch = [&](auto buf, int ks) {
-#pragma unroll
-    for (int e = 0; e < FM + FN; ++e) fetch_one(buf, e, ks);
-  };
-  // buffers 0..NBUF-2 <- K-steps 0..NBUF-2; K-step NBUF-1 is requested by the first step of the loop
-  fetch(std::integral_constant<int, 0>{}, 0);
-  if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
-
-  write_row_tables(lds, my_w, my_a);
-
-  f32x16 acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; ++i)
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-  __syncthreads();
-
-  // ---- main loop: software pipeline over "phases" (one MFMA k-slice of 16) -------
-  // While the matrix core works on the operands looked up in the previous phase, the
-  // wavefront issues the table lookups for the next one.  The instruction order is fixed by
-  // hand: after every MFMA come kLook lookups (address arithmetic + LDS read), and nothing
-  // may be moved across the boundary between two such groups, so the matrix core never
-  // waits behind a burst of lookups and the LDS queue never runs dry.  The first phase of a
-  // K-step also carries the FM+FN global loads of the K-step NBUF-1 ahead, one per group.
-  //
-  // One-code-per-byte activations take two lookups per operand dword (single-code table, the
-  // value in both halves); the two are merged with one v_perm_b32 when the operand is used.
-  constexpr int kRA = AM == A_NIBBLE ? 4 : 8;  // LDS reads per activation tile and phase
-  constexpr int kLookups = kRA * FM + 4 * FN, kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
-  constexpr int kLook = (kLookups + kGroups - 1) / kGroups;
-  uint32_t oa[2][FM][kRA], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
-
-  // dword d (0..7 for bytes, 0..3 for nibbles) of this lane's activation run in buffer B, tile i
-  auto a_word = [&](auto buf, int i, int d) -> uint32_t {
-    constexpr int B = decltype(buf)::value;
-    const uint4 v = pa[B][i][d >> 2];
-    return (d & 3) == 0 ? v.x : (d & 3) == 1 ? v.y : (d & 3) == 2 ? v.z : v.w;
-  };
-  // Lookup t of a phase, in the order the MFMAs of the next phase want their operands:
-  // activation tile 0, every weight tile, then activation tiles 1..FM-1.  Split in two halves
-  // so that the address of a lookup is computed one group before its LDS read is issued.
-  auto lookup_address = [&](auto buf, int q, int t) -> uint32_t {
-    constexpr int B = decltype(buf)::value;
-    const bool is_a = t < kRA || t >= kRA + 4 * FN;
-    if (is_a) {
-      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
-      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
-      if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
-      else return row_address(a_word(buf, i, 2 * q + (sub >> 2)), a_off, sub & 3);  // byte 8q + sub of the run
-    }
-    const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
-    if constexpr (BITS == 4) return row_address(pw[B][j][q], w_off, p);
-    else return 0u;
-  };
-  auto lookup_read = [&](auto buf, int q, int set, int t, uint32_t address) {
-    constexpr int B = decltype(buf)::value;
-    const bool is_a = t < kRA || t >= kRA + 4 * FN;
-    if (is_a) {
-      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
-      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
-      oa[set][i][sub] = lds_read_u32(address);
-    } else {
-      const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
-      if constexpr (BITS == 4) ob[set][j][p] = lds_read_u32(address);
-      else ob[set][j][p] = decode_w_piece<BITS, 6>(pw[B][j], q, p, w_off);
-    }
-  };
-  // the activation operand of tile i out of `set`
-  auto a_operand = [&](int set, int i) -> uint4 {
-    if constexpr (AM == A_NIBBLE) {
-      return make_uint4(oa[set][i][0], oa[set][i][1], oa[set][i][2], oa[set][i][3]);
-    } else {
-      return make_uint4(__builtin_amdgcn_perm(oa[set][i][1], oa[set][i][0], 0x07060100u),
-                        __builtin_amdgcn_perm(oa[set][i][3], oa[set][i][2], 0x07060100u),
-                        __builtin_amdgcn_perm(oa[set][i][5], oa[set][i][4], 0x07060100u),
-                        __builtin_amdgcn_perm(oa[set][i][7], oa[set][i][6], 0x07060100u));
-    }
-  };
-  // lookups of (buf, q) into `set` interleaved with the MFMAs on the other set
-  auto phase = [&](auto buf, int q, int set, auto fetch_buf, int fetch_ks, bool with_fetch) {
-    uint32_t addr[2][kLook];
-    uint4 av = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-    for (int t = 0; t < kLookups / kGroups; ++t) addr[0][t] = lookup_address(buf, q, t);
-#pragma unroll
-    for (int m = 0; m < kGroups; ++m) {
-      const int i = m / FN, j = m % FN;
-      if (j == 0) av = a_operand(set ^ 1, i);
-      const int lo = m * kLookups / kGroups, hi = (m + 1) * kLookups / kGroups, hi2 = (m + 2) * kLookups / kGroups;
-      if (with_fetch && m < FM + FN) fetch_one(fetch_buf, m, fetch_ks);
-      const uint4 bw = make_uint4(ob[set ^ 1][j][0], ob[set ^ 1][j][1], ob[set ^ 1][j][2], ob[set ^ 1][j][3]);
-      // weights first: the accumulator tile is the transposed output tile
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, av),
-                                                          acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int t = lo; t < hi; ++t) lookup_read(buf, q, set, t, addr[m & 1][t - lo]);
-      if (m + 1 < kGroups) {
-#pragma unroll
-        for (int t = hi; t < hi2; ++t) addr[(m + 1) & 1][t - hi] = lookup_address(buf, q, t);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-  // one K-step out of buffer B; its last phase looks up the first operands of buffer B+1
-  auto step = [&](auto buf, int ks) {
-    constexpr int B = decltype(buf)::value;
-    constexpr auto prev = std::integral_constant<int, (B + NBUF - 1) % NBUF>{};
-    constexpr auto next = std::integral_constant<int, (B + 1) % NBUF>{};
-    phase(buf, 1, 1, prev, ks + NBUF - 1, FM + FN <= FM * FN);
-    if constexpr (FM + FN > FM * FN) fetch(prev, ks + NBUF - 1);
-    phase(buf, 2, 0, prev, 0, false);
-    phase(buf, 3, 1, prev, 0, false);
-    phase(next, 0, 0, prev, 0, false);
-  };
-
-#pragma unroll
-  for (int t = 0; t < kLookups; ++t)
-    lookup_read(std::integral_constant<int, 0>{}, 0, 0, t, lookup_address(std::integral_constant<int, 0>{}, 0, t));
-  int ks = 0;
-  for (; ks + NBUF <= steps; ks += NBUF) {
-    step(std::integral_constant<int, 0>{}, ks);
-    step(std::integral_constant<int, 1>{}, ks + 1);
-    if constexpr (NBUF == 3) step(std::integral_constant<int, 2>{}, ks + 2);
-  }
-  if (ks < steps) {
-    step(std::integral_constant<int, 0>{}, ks);
-    if (NBUF == 3 && ks + 1 < steps) step(std::integral_constant<int, 1>{}, ks + 1);
-  }
-
-  __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused from here on
-  if constexpr (KSPLIT == 1) {
-    gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, wn, TN, tid, g.M, g.N,
-                          g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out, g.out_dtype,
-                          reinterpret_cast<unsigned char *>(lds));
-  } else {
-    // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
-    // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
-    // its own slice w.  Slot of destination s: [FN tiles][4 runs][64 lanes] of float4.
-    float4 *slots = reinterpret_cast<float4 *>(lds);
-    auto finish = [&](auto wt) {
-      constexpr int W = decltype(wt)::value;
-#pragma unroll
-      for (int d = 1; d < 4; ++d) {
-        const int dst = (W + d) & 3;
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4)
-            slots[((dst * FN + j) * 4 + a4) * 64 + lane] = make_float4(acc[dst][j][4 * a4 + 0], acc[dst][j][4 * a4 + 1],
-                                                                       acc[dst][j][4 * a4 + 2], acc[dst][j][4 * a4 + 3]);
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            const float4 v = slots[((W * FN + j) * 4 + a4) * 64 + lane];
-            acc[W][j][4 * a4 + 0] += v.x;
-            acc[W][j][4 * a4 + 1] += v.y;
-            acc[W][j][4 * a4 + 2] += v.z;
-            acc[W][j][4 * a4 + 3] += v.w;
-          }
-        __syncthreads();
-      }
-      EpiFactors<1> mine;
-      mine.rn = epi.rn;
-      mine.bv = epi.bv;
-      mine.sc[0] = epi.sc[W];
-      const f32x16 (&slice)[1][FN] = *reinterpret_cast<const f32x16 (*)[1][FN]>(&acc[W]);
-      gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * W, 0, TN, tid, g.M,
-                           g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
-                           reinterpret_cast<unsigned char *>(lds), TM);
-    };
-    if (wave == 0) finish(std::integral_constant<int, 0>{});
-    else if (wave == 1) finish(std::integral_constant<int, 1>{});
-    else if (wave == 2) finish(std::integral_constant<int, 2>{});
-    else finish(std::integral_constant<int, 3>{});
-  }
-}
-
-template <int AM, int BITS, int FM, int FN, int KSPLIT = 1>
-int launch_cfg(GemmArgs g, hipStream_t stream) {
-  constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
-  g.tiles_m = static_cast<int>((g.M + TM - 1) / TM);
-  g.tiles_n = static_cast<int>((g.N + TN - 1) / TN);
-  const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
-  if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
-  auto kern = packed_gemm_kernel<AM, BITS, FM, FN, KSPLIT>;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), 0, stream, g);
-  return check_launch("packed_gemm");
-}
-
-template <int AM, int BITS>
-int launch_bits(const GemmArgs &g, int tile, hipStream_t stream) {
-  if (tile == 4) return launch_cfg<AM, BITS, 4, 3, 4>(g, stream);
-  if (tile == 3) return launch_cfg<AM, BITS, 4, 3>(g, stream);
-  if constexpr (AM == A_NIBBLE) {
-    if (tile == 2) return launch_cfg<AM, BITS, 4, 4>(g, stream);
-  } else {
-    if (tile == 2) return launch_cfg<AM, BITS, 4, 3>(g, stream);  // byte codes need more registers: 256x192 at most
-  }
-  if (tile == 1) return launch_cfg<AM, BITS, 2, 4>(g, stream);
-  return launch_cfg<AM, BITS, 2, 2>(g, stream);
-}
-
-template <int AM>
-int launch_mode(const GemmArgs &g, int bits, int tile, hipStream_t stream) {
-  switch (bits) {
-    case 2: return launch_bits<AM, 2>(g, tile, stream);
-    case 3: return launch_bits<AM, 3>(g, tile, stream);
-    case 4: return launch_bits<AM, 4>(g, tile, stream);
-    case 6: return launch_bits<AM, 6>(g, tile, stream);
-    case 8: return launch_bits<AM, 8>(g, tile, stream);
-    default: return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: weight width %d", bits);
-  }
-}
-
-}  // namespace
+int gemm_launch_bytes(const GemmArgs &g, int bits, int tile, hipStream_t stream);  // packed_gemm_bytes.hip
 
 // Tile choice by a small cost model: a launch runs in `rounds` of as many workgroups as fit
 // on the chip at once; a workgroup costs a fixed prologue + epilogue and a time per K-step
@@ -412,7 +58,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
   const int tile = gemm_choose_tile(M, N, K);
   if (a_mode == A_NIBBLE) return launch_mode<A_NIBBLE>(g, bits, tile, stream);
-  if (a_mode == A_U8) return launch_mode<A_U8>(g, bits, tile, stream);
+  if (a_mode == A_U8) return gemm_launch_bytes(g, bits, tile, stream);
   return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
 }
 
