@@ -52,7 +52,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream);
-int gemm_choose_tile(int64_t M, int64_t N, int64_t K);
+int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits);
 bool gemm_av_supported(int64_t K, int bits);
 int gemm_av_dispatch(bool f16, const void *a, const float *row_scale, const uint8_t *w, int bits,
                      const uint16_t *row_norms, const float *w_cents, const void *bias, int bias_dtype,
@@ -141,7 +141,7 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   hipStream_t s = as_stream(stream);
   if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
     return gemm_av_dispatch(x_dtype == OQ_F16, x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype,
-                            M, N, K, out, out_dtype, gemm_choose_tile(M, N, K), s);
+                            M, N, K, out, out_dtype, gemm_choose_tile(M, N, K, bits), s);
   return generic_matmul_float(x, x_dtype, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N,
                               K, out, out_dtype, s);
 }
