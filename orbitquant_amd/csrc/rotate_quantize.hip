@@ -241,10 +241,16 @@ __device__ __forceinline__ void load_perm_signs(const RqArgs &a, int64_t c0, Per
 }
 
 template <int DT, bool VEC, int LOG_G>
-__global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
+__global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   using Stage = RqStage<DT, VEC, LOG_G>;
-  const int t = threadIdx.x;
+  // Thread = (virtual lane t of the 256-lane pass structure, pass group pg).  With one group a
+  // thread walks all passes of its lane; when few rows are in flight the launcher starts up to
+  // four groups so that the passes of a long row run side by side (group pg takes passes
+  // pg, pg + groups, ...).
+  const int tid = threadIdx.x;
+  const int t = tid & (kThreads - 1);
+  const int pg = tid >> 8, groups_n = blockDim.x > kThreads ? blockDim.x >> 8 : 1;
   const int lane = t & 63;
   const int wave = t >> 6;
   const int64_t row = blockIdx.x;
@@ -258,24 +264,25 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   float *xbuf = reinterpret_cast<float *>(cells_bad + 4);       // Kp elements of Stage::kBytes
   uint16_t *xbuf16 = reinterpret_cast<uint16_t *>(xbuf);
   uint8_t *cbuf = reinterpret_cast<uint8_t *>(xbuf) + static_cast<size_t>(Kp) * Stage::kBytes;  // Kp bytes, big-block path only
+  float *psum = reinterpret_cast<float *>(cbuf + (LOG_G > 0 ? Kp : 0));  // [passes][256], only with several pass groups
 
   // Permutation and signs of the first pass: requested before anything else so their latency
   // overlaps the row load (loads of one wavefront return in order).
   PermSigns ps_cur, ps_nxt;
-  if constexpr (VEC) load_perm_signs(a, static_cast<int64_t>(t) * kChunk, ps_cur);
+  if constexpr (VEC) load_perm_signs(a, static_cast<int64_t>(pg) * kPass + t * kChunk, ps_cur);
 
   // tables
-  const int nthreads = blockDim.x;  // 64 * (wavefronts that own a part of the row), at most 256
-  for (int i = t; i < 256; i += nthreads) {
+  const int nthreads = blockDim.x;  // 64 * (wavefronts that own a part of the row), or 256 * pass groups
+  for (int i = tid; i < 256; i += nthreads) {
     bnd[i] = (i < a.levels - 1) ? a.bounds[i] : __builtin_inff();
     cent[i] = (a.cents != nullptr && i < a.levels) ? a.cents[i] : 0.0f;
   }
-  if (t == 0) cells_bad[0] = 0;
+  if (tid == 0) cells_bad[0] = 0;
 
   // ---- phase A: stage the row, sum of squares in the documented order --------
   const int64_t row_base = row * K;
   float q = 0.0f;
-  for (int p = 0; p < a.passes; ++p) {
+  for (int p = pg; p < a.passes; p += groups_n) {
     const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
     float f[kChunk];
     if constexpr (Stage::k16) {
@@ -303,7 +310,15 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
 #pragma unroll
     for (int e = 0; e < kChunk; ++e) s[e] = f[e] * f[e];
     const float v8 = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
-    q = (p == 0) ? v8 : q + v8;
+    if (groups_n == 1) q = (p == 0) ? v8 : q + v8;
+    else psum[p * kThreads + t] = v8;
+  }
+  if (groups_n > 1) {  // the lane's passes were summed by different threads: add them left to right
+    __syncthreads();
+    if (pg == 0) {
+      q = psum[t];
+      for (int p = 1; p < a.passes; ++p) q = q + psum[p * kThreads + t];
+    }
   }
   q = q + lane_xor<1>(q);
   q = q + lane_xor<2>(q);
@@ -311,15 +326,15 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   q = q + lane_xor<8>(q);
   q = q + lane_xor<16>(q);
   q = q + lane_xor<32>(q);
-  if (lane == 0) red[wave] = q;
+  if (lane == 0 && pg == 0) red[wave] = q;
   __syncthreads();
-  const int nwaves = nthreads >> 6;  // wavefronts that were not launched own only padding: their sum is 0
+  const int nwaves = min(nthreads, kThreads) >> 6;  // wavefronts that were not launched own only padding: their sum is 0
   const float total = (red[0] + (nwaves > 1 ? red[1] : 0.0f)) + ((nwaves > 2 ? red[2] : 0.0f) + (nwaves > 3 ? red[3] : 0.0f));
   const float s_norm = sqrtf(total);  // IEEE-rounded (hipcc's default for fp32 sqrt and division)
   const float denom = s_norm + a.eps;
   const float recip = 1.0f / denom;
   const bool row_plain = !(denom > 1e-30f && denom < 1e30f);  // the reciprocal itself would lose bits
-  if (t == 0 && a.norms != nullptr) a.norms[row] = s_norm;
+  if (tid == 0 && a.norms != nullptr) a.norms[row] = s_norm;
 
   // ---- bucketize table (the boundaries are in LDS since the barrier above) ----------------
   CellMap cmap;
@@ -332,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   }
   if (cmap.cells > 0) {
     const int nb = a.levels - 1;
-    for (int c = t; c < cmap.cells; c += nthreads) {
+    for (int c = tid; c < cmap.cells; c += nthreads) {
       // boundaries are ascending, so their cells are too: first boundary with cell >= c, first with cell > c
       int first = 0, last = 0;
       for (int step = a.levels_pow2; step > 0; step >>= 1) {
@@ -364,13 +379,14 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
   float keep[BIG ? kMaxPasses : 1][kChunk];
 
 #pragma unroll
-  for (int p = 0; p < kMaxPasses; ++p) {
+  for (int pi = 0; pi < kMaxPasses; ++pi) {
+    const int p = pg + pi * groups_n;
     // small blocks: a wavefront whose 512 slots of this pass all lie past the row has nothing to do
     if (p < a.passes && (BIG || static_cast<int64_t>(p) * kPass + (t & ~63) * kChunk < K)) {
       const int64_t c0 = static_cast<int64_t>(p) * kPass + t * kChunk;
       float y[kChunk];
       if constexpr (VEC) {
-        if (p + 1 < a.passes) load_perm_signs(a, c0 + kPass, ps_nxt);  // one pass ahead
+        if (p + groups_n < a.passes) load_perm_signs(a, c0 + static_cast<int64_t>(groups_n) * kPass, ps_nxt);  // one pass ahead
       }
       if (VEC && c0 + kChunk <= K) {
         const int idx[kChunk] = {ps_cur.pa.x, ps_cur.pa.y, ps_cur.pa.z, ps_cur.pa.w,
@@ -424,7 +440,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
         if (c0 < K) emit8<DT, VEC>(a, row, c0, code, cent, s_norm);
       } else {
 #pragma unroll
-        for (int e = 0; e < kChunk; ++e) keep[p][e] = y[e];
+        for (int e = 0; e < kChunk; ++e) keep[pi][e] = y[e];
       }
     }
   }
@@ -433,17 +449,18 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
     // ---- phase C: distances 512 .. block/2 through LDS --------------------------
     __syncthreads();  // every gather has read xbuf
 #pragma unroll
-    for (int p = 0; p < kMaxPasses; ++p) {
+    for (int pi = 0; pi < kMaxPasses; ++pi) {
+      const int p = pg + pi * groups_n;
       if (p < a.passes) {
         float4 *dst = reinterpret_cast<float4 *>(xbuf + static_cast<int64_t>(p) * kPass + t * kChunk);
-        dst[0] = make_float4(keep[p][0], keep[p][1], keep[p][2], keep[p][3]);
-        dst[1] = make_float4(keep[p][4], keep[p][5], keep[p][6], keep[p][7]);
+        dst[0] = make_float4(keep[pi][0], keep[pi][1], keep[pi][2], keep[pi][3]);
+        dst[1] = make_float4(keep[pi][4], keep[pi][5], keep[pi][6], keep[pi][7]);
       }
     }
     __syncthreads();
     constexpr int G = 1 << LOG_G;  // block / 512
     const int groups = static_cast<int>(K >> LOG_G);
-    for (int gi = t; gi < groups; gi += nthreads) {
+    for (int gi = tid; gi < groups; gi += nthreads) {
       const int base = (gi >> 9) * h + (gi & (kLaneSpan - 1));
       float z[G];
 #pragma unroll
@@ -454,7 +471,7 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
         cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(code_of(z[v] * a.inv_sqrt_block));
     }
     __syncthreads();
-    for (int64_t c0 = t * kChunk; c0 < K; c0 += kPass) {
+    for (int64_t c0 = static_cast<int64_t>(tid) * kChunk; c0 < K; c0 += static_cast<int64_t>(max(nthreads, kThreads)) * kChunk) {
       const uint2 w = *reinterpret_cast<const uint2 *>(cbuf + c0);
       int code[kChunk];
 #pragma unroll
@@ -465,12 +482,15 @@ __global__ __launch_bounds__(kThreads) void rotate_quantize_kernel(RqArgs a) {
 }
 
 template <int DT, bool VEC>
-int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {
+int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {  // smem: bytes without the pass-group scratch
   int log_g = 0;
   for (int g = a.block / kLaneSpan; g > 1; g >>= 1) ++log_g;
   // a wavefront owns 512 consecutive elements of a pass: launch only the wavefronts a single-pass row needs
   const int waves = a.K >= 3 * kLaneSpan ? 4 : static_cast<int>((a.K + kLaneSpan - 1) / kLaneSpan);
-  dim3 grid(static_cast<unsigned>(a.M)), block(64 * waves);
+  // few rows (decode): the chip is empty anyway, so run the passes of a long row side by side
+  const int pass_groups = (a.M <= 64 && a.passes >= 2 && getenv("OQ_RQ_ONE_GROUP") == nullptr) ? (a.passes >= 3 ? 4 : 2) : 1;
+  dim3 grid(static_cast<unsigned>(a.M)), block(pass_groups > 1 ? kThreads * pass_groups : 64 * waves);
+  if (pass_groups > 1) smem += static_cast<size_t>(a.passes) * kThreads * sizeof(float);
 #define OQ_RQ_CASE(LG)                                                                           \
   case LG: {                                                                                     \
     auto kern = rotate_quantize_kernel<DT, VEC, LG>;                                             \
