@@ -118,8 +118,13 @@ __device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN],
     unsigned char *dst = static_cast<unsigned char *>(out) + m_first * row_pitch + nn * ES;
     const int rows_left = static_cast<int>(min(static_cast<int64_t>(FM * 32), M - m_first));  // rows m_first+k, k < rows_left, exist
     const bool col_ok = nn < N;
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
+    // Software pipeline over the row tiles: the staging writes and read-backs of tile i are issued
+    // before the arithmetic and stores of tile i-1, so LDS latency hides behind them (LDS
+    // operations of a wavefront execute in order, so re-using the one staging tile is safe).
+    constexpr int kReads = 4;  // read instructions per tile at most (32 / RPI with RPI >= 8)
+    float4 v0[2][kReads], v1[2][kReads];
+    float sc[2][kReads];
+    auto stage = [&](int i, int buf) {
 #pragma unroll
       for (int jj = 0; jj < JC; ++jj)
 #pragma unroll
@@ -132,12 +137,19 @@ __device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN],
 #pragma unroll
       for (int t = 0; t < 32 / RPI; ++t) {
         const int row = t * RPI + row0;
-        const float4 v0 = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32);
-        const float4 v1 = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32 + 16);
-        const float sc = sc_s[wm + 32 * i + row];
-        const float y[8] = {(v0.x * sc) * rn0.x + bv0.x, (v0.y * sc) * rn0.y + bv0.y, (v0.z * sc) * rn0.z + bv0.z,
-                            (v0.w * sc) * rn0.w + bv0.w, (v1.x * sc) * rn1.x + bv1.x, (v1.y * sc) * rn1.y + bv1.y,
-                            (v1.z * sc) * rn1.z + bv1.z, (v1.w * sc) * rn1.w + bv1.w};
+        v0[buf][t] = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32);
+        v1[buf][t] = *reinterpret_cast<const float4 *>(tile + row * kEpiPitch + c * 32 + 16);
+        sc[buf][t] = sc_s[wm + 32 * i + row];
+      }
+    };
+    auto finish = [&](int i, int buf) {
+#pragma unroll
+      for (int t = 0; t < 32 / RPI; ++t) {
+        const float4 a0 = v0[buf][t], a1 = v1[buf][t];
+        const float s = sc[buf][t];
+        const float y[8] = {(a0.x * s) * rn0.x + bv0.x, (a0.y * s) * rn0.y + bv0.y, (a0.z * s) * rn0.z + bv0.z,
+                            (a0.w * s) * rn0.w + bv0.w, (a1.x * s) * rn1.x + bv1.x, (a1.y * s) * rn1.y + bv1.y,
+                            (a1.z * s) * rn1.z + bv1.z, (a1.w * s) * rn1.w + bv1.w};
         if (!GUARD || (col_ok && 32 * i + t * RPI < rows_left)) {
           unsigned char *o = dst + (32 * i + t * RPI) * row_pitch;
           if constexpr (OUT_DT == OQ_F32) {
@@ -149,7 +161,14 @@ __device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN],
           }
         }
       }
+    };
+    stage(0, 0);
+#pragma unroll
+    for (int i = 1; i < FM; ++i) {
+      stage(i, i & 1);
+      finish(i - 1, (i - 1) & 1);
     }
+    finish(FM - 1, (FM - 1) & 1);
   }
 }
 
