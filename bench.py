@@ -209,7 +209,8 @@ def _code_format(layer, x):
     """The activation-code format OrbitLinear's forward picks for this input (orbitquant_amd/layers.py)."""
     if layer.activation_bits <= 4:
         return "nibble"
-    return "u8" if x.numel() // layer.in_features > 16 and layer.in_features % 64 == 0 else None
+    tokens, k = x.numel() // layer.in_features, layer.in_features
+    return "u8" if (tokens > 16 and k % 64 == 0) or k % 128 == 0 else None
 
 
 def gemm_only_closure(layer, x):

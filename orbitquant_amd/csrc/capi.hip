@@ -58,7 +58,7 @@ int gemm_av_dispatch(bool f16, const void *a, const float *row_scale, const uint
                      const uint16_t *row_norms, const float *w_cents, const void *bias, int bias_dtype,
                      int64_t M, int64_t N, int64_t K, void *out, int out_dtype, int tile, hipStream_t stream);
 bool gemv_supported(int64_t M, int64_t K, int bits, int code_format, int a_levels);
-int gemv_dispatch(const void *codes, const float *row_scale, const float *act_cents, int a_levels,
+int gemv_dispatch(const void *codes, int code_format, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream);
@@ -122,7 +122,7 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
   const bool fast_ptrs = aligned16(codes) && aligned16(packed_w);
   const bool tiled_out = gemm_output_ok(N, out);  // the tiled kernels store 16-byte row segments
   if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
-    return gemv_dispatch(codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
+    return gemv_dispatch(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
   if (fast_ptrs && tiled_out && gemm_supported(K, w_bits) && (code_format == OQ_CODES_NIBBLE || M > 16))
     return gemm_dispatch(code_format == OQ_CODES_NIBBLE ? 0 : 1, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,

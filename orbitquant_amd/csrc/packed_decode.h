@@ -166,20 +166,30 @@ __device__ __forceinline__ float lane_table(const float *__restrict__ cents, int
 
 // Build the block with WAVES wavefronts: wavefront w writes rows [w*256/WAVES, (w+1)*256/WAVES),
 // four rows per 16-byte-per-lane store.  The caller puts a barrier between this and the first lookup.
-template <int BITS, int WAVES>
+// A_SINGLE: the activation half holds single-code entries (one code per byte, up to 256 levels)
+// instead of the pair table of two 4-bit codes.
+template <int BITS, int WAVES, bool A_SINGLE = false>
 __device__ __forceinline__ void build_row_tables(uint32_t *lds, const float *__restrict__ w_cents,
                                                  const float *__restrict__ act_cents, int a_levels) {
   constexpr int kLevels = 1 << BITS;
   constexpr bool kPair = BITS <= 4;
   constexpr int kRowsPerWave = 256 / WAVES;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const float a_tab = lane_table<16>(act_cents, a_levels);
+  const float a_tab = A_SINGLE ? lane_table<64>(act_cents, a_levels) : lane_table<16>(act_cents, a_levels);
   float w_tab = 0.0f;
   if constexpr (kLevels <= 64) w_tab = lane_table<kLevels>(w_cents, kLevels);
 #pragma unroll
   for (int i = 0; i < kRowsPerWave / 4; ++i) {
     const int e = wave * kRowsPerWave + 4 * i + (lane >> 4);  // the row this lane writes to
-    const uint32_t ea = pack16(__shfl(a_tab, e & 15), __shfl(a_tab, e >> 4), false);
+    uint32_t ea;
+    if constexpr (A_SINGLE) {
+      float v = __shfl(a_tab, e & 63);
+      if (a_levels > 64) v = e < a_levels ? act_cents[e] : 0.0f;  // wide tables: one vector load per row
+      else if (e >= a_levels) v = 0.0f;
+      ea = pack16(v, v, false);
+    } else {
+      ea = pack16(__shfl(a_tab, e & 15), __shfl(a_tab, e >> 4), false);
+    }
     uint32_t ew;
     if constexpr (kLevels <= 64) {
       if constexpr (kPair) {

@@ -29,7 +29,7 @@ namespace oq {
 namespace {
 
 struct GemvArgs {
-  const uint8_t *a;          // nibble codes [M, K/2]
+  const uint8_t *a;          // activation codes: [M, K/2] two per byte, or [M, K] one per byte
   const float *row_scale;    // [M] or NULL
   const float *act_cents;
   int a_levels;
@@ -47,8 +47,11 @@ struct GemvArgs {
 constexpr int kDepth = 1;  // K-steps of 128 fetched per batch of global loads (two batches in flight: decode of one overlaps the stream of the next)
 constexpr int kGemvTableBytes = kRowTableBytes;
 
-template <int BITS, int R, int WAVES>
+// BYTES: activation codes come one per byte (widths above 4 bits) instead of two per byte.
+template <bool BYTES, int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
+  constexpr int kAVec = BYTES ? 2 : 1;      // 16-byte loads of activation codes per lane and K-step
+  constexpr int kAStep = 64 * kAVec;        // bytes of one activation row per K-step of 128
   static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
   __shared__ __attribute__((aligned(65536))) uint32_t lds[kGemvTableBytes / 4];
   float *partial = reinterpret_cast<float *>(lds);  // [WAVES][R][64][4], after the main loop
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   const int s_end = static_cast<int>(static_cast<int64_t>(steps) * (wave + 1) / WAVES);
 
   const int64_t w_row_bytes = g.K * BITS / 8;
-  const uint8_t *ap = g.a + static_cast<int64_t>(min(r, g.M - 1)) * (g.K / 2) + grp * 16;
+  const uint8_t *ap = g.a + static_cast<int64_t>(min(r, g.M - 1)) * (BYTES ? g.K : g.K / 2) + grp * (16 * kAVec);
   const uint8_t *wp[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) {
@@ -74,14 +77,16 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
 
   // a batch = kDepth K-steps: every load of the batch is issued before anything waits on it
   struct Batch {
-    uint4 a[kDepth];
+    uint4 a[kDepth][kAVec];
     uint32_t w[kDepth][R][BITS];
   };
   auto fetch = [&](int s0, Batch &bt) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       const int s = min(s0 + d, s_end - 1);  // clamped: stays inside the row, result unused
-      bt.a[d] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * 64);
+#pragma unroll
+      for (int v = 0; v < kAVec; ++v)
+        bt.a[d][v] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * kAStep + 16 * v);
 #pragma unroll
       for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s) * (16 * BITS), bt.w[d][j]);
     }
@@ -96,8 +101,16 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
       if (s0 + d < s_end) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t f = q == 0 ? bt.a[d].x : q == 1 ? bt.a[d].y : q == 2 ? bt.a[d].z : bt.a[d].w;
-          const uint4 af = decode_bytes(f, a_off);
+          uint4 af;
+          if constexpr (!BYTES) {
+            const uint4 v = bt.a[d][0];
+            af = decode_bytes(q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w, a_off);
+          } else {  // eight single-code lookups (value in both halves), merged two by two
+            const uint4 v = bt.a[d][q >> 1];
+            const uint4 e0 = decode_bytes((q & 1) ? v.z : v.x, a_off), e1 = decode_bytes((q & 1) ? v.w : v.y, a_off);
+            af = make_uint4(__builtin_amdgcn_perm(e0.y, e0.x, 0x07060100u), __builtin_amdgcn_perm(e0.w, e0.z, 0x07060100u),
+                            __builtin_amdgcn_perm(e1.y, e1.x, 0x07060100u), __builtin_amdgcn_perm(e1.w, e1.z, 0x07060100u));
+          }
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             uint4 bf;
@@ -131,7 +144,7 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   }
 
   // ---- tables (built while the stream is in flight) ---------------------------------------
-  build_row_tables<BITS, WAVES>(lds, g.w_cents, g.act_cents, g.a_levels);
+  build_row_tables<BITS, WAVES, BYTES>(lds, g.w_cents, g.act_cents, g.a_levels);
   __syncthreads();
 
   for (int s = s_begin; s < s_end; s += 2 * kDepth) {
@@ -169,23 +182,25 @@ __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   }
 }
 
-template <int BITS, int R, int WAVES>
+template <bool BYTES, int BITS, int R, int WAVES>
 int launch(const GemvArgs &g, hipStream_t stream) {
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
   if (groups > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: N too large");
-  auto kern = packed_gemv_kernel<BITS, R, WAVES>;
+  auto kern = packed_gemv_kernel<BYTES, BITS, R, WAVES>;
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), 0, stream, g);
   return check_launch("packed_gemv");
 }
 
-template <int BITS, int R>
+template <bool BYTES, int BITS, int R>
 int launch_waves(const GemvArgs &g, int waves, hipStream_t stream) {
-  if (waves == 4) return launch<BITS, R, 4>(g, stream);
-  if (waves == 16) return launch<BITS, R, 16>(g, stream);
-  return launch<BITS, R, 8>(g, stream);
+  if constexpr (!BYTES) {  // the other wavefront counts exist for experiments with OQ_GEMV_CFG only
+    if (waves == 4) return launch<BYTES, BITS, R, 4>(g, stream);
+    if (waves == 16) return launch<BYTES, BITS, R, 16>(g, stream);
+  }
+  return launch<BYTES, BITS, R, 8>(g, stream);
 }
 
-template <int BITS>
+template <bool BYTES, int BITS>
 int launch_bits(const GemvArgs &g, hipStream_t stream) {
   // rows per workgroup (16*R) and K-split (wavefronts per workgroup); OQ_GEMV_CFG="R,WAVES" overrides
   int r = g.N <= 16 * 512 ? 1 : 2, waves = 8;
@@ -196,19 +211,21 @@ int launch_bits(const GemvArgs &g, hipStream_t stream) {
       waves = cw;
     }
   }
-  if (r == 1) return launch_waves<BITS, 1>(g, waves, stream);
-  if (r == 4) return launch_waves<BITS, 4>(g, waves, stream);
-  return launch_waves<BITS, 2>(g, waves, stream);
+  if (r == 1) return launch_waves<BYTES, BITS, 1>(g, waves, stream);
+  if constexpr (!BYTES) {
+    if (r == 4) return launch_waves<BYTES, BITS, 4>(g, waves, stream);
+  }
+  return launch_waves<BYTES, BITS, 2>(g, waves, stream);
 }
 
 }  // namespace
 
 bool gemv_supported(int64_t M, int64_t K, int bits, int code_format, int a_levels) {
-  return M >= 1 && M <= 16 && K % 128 == 0 && code_format == OQ_CODES_NIBBLE && a_levels <= 16 &&
-         (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
+  const bool codes_ok = code_format == OQ_CODES_NIBBLE ? a_levels <= 16 : a_levels <= 256;
+  return M >= 1 && M <= 16 && K % 128 == 0 && codes_ok && (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
 }
 
-int gemv_dispatch(const void *codes, const float *row_scale, const float *act_cents, int a_levels,
+int gemv_dispatch(const void *codes, int code_format, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream) {
@@ -216,14 +233,18 @@ int gemv_dispatch(const void *codes, const float *row_scale, const float *act_ce
   g.a = static_cast<const uint8_t *>(codes); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = static_cast<int>(M); g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
-  switch (bits) {
-    case 2: return launch_bits<2>(g, stream);
-    case 3: return launch_bits<3>(g, stream);
-    case 4: return launch_bits<4>(g, stream);
-    case 6: return launch_bits<6>(g, stream);
-    case 8: return launch_bits<8>(g, stream);
-    default: return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: weight width %d", bits);
+#define OQ_GEMV_BITS(BYTES)                                                   \
+  switch (bits) {                                                             \
+    case 2: return launch_bits<BYTES, 2>(g, stream);                          \
+    case 3: return launch_bits<BYTES, 3>(g, stream);                          \
+    case 4: return launch_bits<BYTES, 4>(g, stream);                          \
+    case 6: return launch_bits<BYTES, 6>(g, stream);                          \
+    case 8: return launch_bits<BYTES, 8>(g, stream);                          \
+    default: return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: weight width %d", bits); \
   }
+  if (code_format == OQ_CODES_NIBBLE) { OQ_GEMV_BITS(false) }
+  OQ_GEMV_BITS(true)
+#undef OQ_GEMV_BITS
 }
 
 }  // namespace oq

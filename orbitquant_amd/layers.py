@@ -55,8 +55,8 @@ def quantized_linear_forward(
             code_format="nibble", activation_bits=activation_bits, weight_bits=weight_bits,
             out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
     tokens = x.numel() // in_features
-    if tokens > 16 and in_features % 64 == 0:
-        # wider activation codes, many tokens: one code per byte into the all-table tile kernel
+    if (tokens > 16 and in_features % 64 == 0) or in_features % 128 == 0:
+        # wider activation codes: one code per byte into the all-table tile / streaming kernels
         codes, _, norms = ops.rotate_quantize(
             x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
             inv_sqrt_block=inv_sqrt_block, code_format="u8")

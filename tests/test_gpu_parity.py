@@ -349,6 +349,20 @@ def test_packed_linear_small_m_stream_kernel(dev, m, n, k, wbits):
     assert torch.equal(got, again)      # fixed summation order: run-to-run identical
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize(("n", "k", "wbits", "abits"), [(2048, 4096, 4, 6), (1000, 1024, 3, 8), (512, 1152, 6, 5), (4096, 4096, 2, 7)])
+def test_packed_linear_small_m_byte_codes(dev, m, n, k, wbits, abits):
+    """Decode-sized inputs with activation codes wider than 4 bits (one code per byte)."""
+    rng = np.random.default_rng(m + n + k + wbits + abits)
+    layer = make_layer(rng, n, k, wbits, abits)
+    _, x32 = make_x(rng, m, k, torch.bfloat16, kind="plain")
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    got = run_packed_linear(dev, layer, codes, s, "u8")
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "small-M byte codes")
+    assert torch.equal(got, run_packed_linear(dev, layer, codes, s, "u8"))
+
+
 # ------------------------------------------------- float-activation packed matmul
 
 def _pack_loop(values, bits):
