@@ -36,6 +36,25 @@ def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+class _OnDevice:
+    """Make `t`'s device current for a launch; free when it already is (the usual case)."""
+
+    __slots__ = ("_guard",)
+
+    def __init__(self, t: torch.Tensor) -> None:
+        index = t.device.index
+        self._guard = None if index is None or index == torch.cuda.current_device() else torch.cuda.device(index)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            return self._guard.__exit__(*exc)
+        return False
+
+
 def rotate_quantize(
     x: torch.Tensor,
     permutation: torch.Tensor,
@@ -88,7 +107,7 @@ def rotate_quantize(
         raise ValueError("centroids are required when values are requested")
     norms = torch.empty(m, dtype=torch.float32, device=x.device)
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _OnDevice(x):
         rc = lib.oq_rotate_quantize(
             rows.data_ptr(), _dt(rows), m, dim, permutation.data_ptr(), signs.data_ptr(),
             boundaries.data_ptr(), _ptr(centroids), levels, int(block_size), float(eps),
@@ -136,7 +155,7 @@ def packed_linear(
     if norms.dtype != torch.float32 or norms.numel() != m:
         raise ValueError("token_norms must be float32 with one entry per token")
     lib = _lib.load()
-    with torch.cuda.device(codes.device):
+    with _OnDevice(codes):
         rc = lib.oq_packed_linear(
             flat.data_ptr(), fmt, norms.contiguous().data_ptr(), activation_centroids.data_ptr(),
             int(activation_bits), packed_weight_indices.data_ptr(), int(weight_bits),
@@ -167,7 +186,7 @@ def matmul_packed_weight_values(
     out_dtype = x.dtype if output_dtype is None else output_dtype
     out = torch.empty((m, out_features), dtype=out_dtype, device=x.device)
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _OnDevice(x):
         rc = lib.oq_matmul_packed_weight(
             flat.data_ptr(), _dt(flat), _ptr(token_scale), packed_weight_indices.data_ptr(), int(bits),
             row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
@@ -181,7 +200,7 @@ def unpack_lowbit(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
     _require_gpu(packed, "packed")
     out = torch.empty(length, dtype=torch.uint8, device=packed.device)
     lib = _lib.load()
-    with torch.cuda.device(packed.device):
+    with _OnDevice(packed):
         rc = lib.oq_unpack_lowbit(packed.contiguous().data_ptr(), int(bits), int(length), out.data_ptr(),
                                   _stream(packed))
     _lib.check(rc, "oq_unpack_lowbit")
