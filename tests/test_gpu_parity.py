@@ -320,6 +320,20 @@ def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
     check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, f"tile {tile}")
 
 
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4"])
+@pytest.mark.parametrize(("m", "n", "k"), [(17, 8, 256), (33, 24, 512), (300, 8, 256)])
+def test_packed_linear_tiny_outputs_every_tile(dev, m, n, k, tile, monkeypatch):
+    """Outputs much smaller than a tile: every row / column clamp and store guard is exercised."""
+    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+    rng = np.random.default_rng(m * 5 + n + k + int(tile))
+    layer = make_layer(rng, n, k, 4, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, torch.float32)
+    got = run_packed_linear(dev, layer, codes, s, "nibble", torch.float32)
+    check_outputs(got.cpu().numpy(), want, s, layer["r"].float().numpy(), k, f"tiny tile {tile}")
+
+
 @pytest.mark.parametrize(("m", "n", "k", "wbits"), [(300, 200, 1024, 4), (128, 96, 256, 4), (515, 1152, 2304, 3), (130, 104, 512, 6)])
 def test_packed_linear_k_split_kernel(dev, m, n, k, wbits, monkeypatch):
     """Four wavefronts share one output tile and a quarter of K each; partial tiles are summed through LDS."""
