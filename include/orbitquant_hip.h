@@ -92,6 +92,29 @@ int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K,
                        float *norms_out, void *stream);
 
 /*
+ * The same, on f(x) instead of x, for an elementwise function f of a 16-bit
+ * input given as a table: input_map[bits of x] = bits of f(x), 65536 entries of
+ * the same dtype as x, 16-byte aligned, on the device.  The result is what
+ * oq_rotate_quantize returns for the tensor f(x), bit for bit; f(x) is never
+ * written to memory.  x_dtype must be OQ_F16 or OQ_BF16.
+ *
+ * No counterpart in the reference's extension: there the activation between two
+ * quantized linears (the GELU of an MLP, functional calls in the model code) is
+ * a separate elementwise kernel that writes f(x) and the quantizer reads it
+ * back; the table is how a caller hands that function to this kernel without
+ * changing its results (fill it by applying the framework's own f to all
+ * 65536 bit patterns).
+ */
+int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_map,
+                              int64_t M, int64_t K,
+                              const int32_t *perm, const int8_t *signs,
+                              const float *boundaries, const float *centroids, int levels,
+                              int64_t block, float eps, float inv_sqrt_block,
+                              void *codes_out, int code_format,
+                              void *values_out, int values_mode,
+                              float *norms_out, void *stream);
+
+/*
  * Packed-weight linear on quantized activations (the fused hot path):
  *
  *   out[m,n] = (sum_k c_a[code[m,k]] * c_w[idx[n,k]]) * s[m] * r_w[n] + bias[n]

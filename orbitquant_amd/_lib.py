@@ -19,8 +19,8 @@ OQ_VALUES_NONE, OQ_VALUES_SCALED, OQ_VALUES_UNIT_BF16 = 0, 1, 2
 _STATUS = {1: "invalid argument", 2: "unsupported", 3: "launch failure"}
 
 EXPORTS = (
-    "oq_device_ok", "oq_last_error", "oq_version", "oq_rotate_quantize", "oq_packed_linear",
-    "oq_matmul_packed_weight", "oq_unpack_lowbit",
+    "oq_device_ok", "oq_last_error", "oq_version", "oq_rotate_quantize", "oq_rotate_quantize_mapped",
+    "oq_packed_linear", "oq_matmul_packed_weight", "oq_unpack_lowbit",
 )
 
 _lib = None
@@ -47,6 +47,9 @@ def load() -> ctypes.CDLL:
     lib.oq_rotate_quantize.restype = c_int
     lib.oq_rotate_quantize.argtypes = [vp, c_int, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f,
                                        vp, c_int, vp, c_int, vp, vp]
+    lib.oq_rotate_quantize_mapped.restype = c_int
+    lib.oq_rotate_quantize_mapped.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f,
+                                              vp, c_int, vp, c_int, vp, vp]
     lib.oq_packed_linear.restype = c_int
     lib.oq_packed_linear.argtypes = [vp, c_int, vp, vp, c_int, vp, c_int, vp, vp, vp, c_int,
                                      c_i64, c_i64, c_i64, vp, c_int, vp]

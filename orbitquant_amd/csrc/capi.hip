@@ -36,7 +36,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              const int8_t *signs, const float *boundaries, const float *centroids,
                              int levels, int64_t block, float eps, float inv_sqrt_block,
                              void *codes_out, int code_format, void *values_out, int values_mode,
-                             float *norms_out, hipStream_t stream);
+                             float *norms_out, const uint16_t *input_map, hipStream_t stream);
 int generic_matmul_float(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
                          int bits, const uint16_t *row_norms, const float *w_cents, const void *bias,
                          int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
@@ -104,7 +104,18 @@ int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K, const i
                        void *values_out, int values_mode, float *norms_out, void *stream) {
   return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
                                   inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
-                                  as_stream(stream));
+                                  nullptr, as_stream(stream));
+}
+
+int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
+                              const int32_t *perm, const int8_t *signs, const float *boundaries,
+                              const float *centroids, int levels, int64_t block, float eps, float inv_sqrt_block,
+                              void *codes_out, int code_format, void *values_out, int values_mode,
+                              float *norms_out, void *stream) {
+  if (input_map == nullptr) return fail(OQ_ERR_INVALID, "rotate_quantize_mapped: input_map is null");
+  return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
+                                  inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
+                                  input_map, as_stream(stream));
 }
 
 int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,

@@ -8,7 +8,7 @@
 // applies the sign and runs the Walsh-Hadamard butterflies:
 //   distance 1,2,4        in registers (the thread's own eight values)
 //   distance 8 .. 256     across the lanes of the wavefront (lane xor 1 .. 32: DPP lane
-//                         exchanges up to 8, wavefront shuffles for 16 and 32)
+//                         exchanges up to 8, wavefront shuffles or lane-group swaps of register pairs for 16 and 32)
 //   distance 512 ..       through LDS, regrouped so the stages are register-local
 // Every butterfly output is one fp32 add or subtract of two values of the
 // previous stage, so the result does not depend on this schedule.
@@ -50,11 +50,63 @@ struct RqArgs {
   void *values;
   int values_mode;
   float *norms;
+  const uint16_t *map;  // optional elementwise map of 16-bit inputs: 65536 entries indexed by the input's bits
+  int map_lo;           // bf16 only: first |bits| of the window of 2 x 2048 entries kept in LDS; < 0: no window
+  int map_lds_offset;   // where the window starts in the dynamic LDS block (bytes, a multiple of 16)
 };
 
+constexpr int kHotHalf = 2048;                  // entries per sign: 16 binades of bf16
+constexpr int kHotBytes = 2 * kHotHalf * 2;     // 8 KB of LDS
+
+// The mapped value of eight 16-bit inputs.  bf16 inputs inside the window (|x| in 16 binades
+// chosen by the launcher, both signs) are served from the copy in LDS; a wavefront with any
+// input outside it also reads the full table in memory for those.  Other dtypes read the full
+// table for every input.
+template <int DT>
+__device__ __forceinline__ uint4 map_raw8(const uint4 raw, const RqArgs &a, const uint16_t *hot) {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t out[4];
+  if (DT == OQ_BF16 && hot != nullptr) {
+    const uint32_t lo2 = static_cast<uint32_t>(a.map_lo) * 0x10001u;
+    uint32_t outside = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // per half: t = bits - lo (16-bit wrap); inside the window <=> (t & 0x7fff) < 2048; slot = (t & 0x7ff) + 2048 * sign
+      const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
+      outside |= t;
+      const uint32_t slot = (t & 0x07ff07ffu) | ((t >> 4) & 0x08000800u);
+      out[j] = static_cast<uint32_t>(hot[slot & 0xffffu]) | (static_cast<uint32_t>(hot[slot >> 16]) << 16);
+    }
+    if (__builtin_amdgcn_ballot_w64((outside & 0x78007800u) != 0) != 0) {
+      // all sixteen-bit loads are issued before any is used; inputs inside the window read entry 0 and drop it
+      uint32_t far[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
+        far[2 * j] = a.map[(t & 0x00007800u) ? (w[j] & 0xffffu) : 0u];
+        far[2 * j + 1] = a.map[(t & 0x78000000u) ? (w[j] >> 16) : 0u];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
+        if (t & 0x00007800u) out[j] = (out[j] & 0xffff0000u) | far[2 * j];
+        if (t & 0x78000000u) out[j] = (out[j] & 0x0000ffffu) | (far[2 * j + 1] << 16);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      out[j] = static_cast<uint32_t>(a.map[w[j] & 0xffffu]) | (static_cast<uint32_t>(a.map[w[j] >> 16]) << 16);
+  }
+  return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
 template <int DT, bool VEC>
-__device__ __forceinline__ void load_chunk(const void *x, int64_t row_base, int64_t i0, int64_t K,
+__device__ __forceinline__ void load_chunk(const RqArgs &a, const uint16_t *hot, int64_t row_base, int64_t i0,
                                            float (&f)[kChunk]) {
+  const void *x = a.x;
+  const int64_t K = a.K;
   if constexpr (VEC) {
     if (i0 + kChunk <= K) {
       if constexpr (DT == OQ_F32) {
@@ -63,7 +115,8 @@ __device__ __forceinline__ void load_chunk(const void *x, int64_t row_base, int6
         f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
         f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
       } else {
-        const uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(x) + row_base + i0);
+        uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(x) + row_base + i0);
+        if (a.map != nullptr) raw = map_raw8<DT>(raw, a, hot);
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -81,7 +134,19 @@ __device__ __forceinline__ void load_chunk(const void *x, int64_t row_base, int6
     }
   }
 #pragma unroll
-  for (int e = 0; e < kChunk; ++e) f[e] = (i0 + e < K) ? load_as_f32<DT>(x, row_base + i0 + e) : 0.0f;
+  for (int e = 0; e < kChunk; ++e) {
+    f[e] = 0.0f;
+    if (i0 + e < K) {
+      if constexpr (DT != OQ_F32) {
+        if (a.map != nullptr) {
+          const uint16_t bits = a.map[static_cast<const uint16_t *>(x)[row_base + i0 + e]];
+          f[e] = DT == OQ_BF16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+          continue;
+        }
+      }
+      f[e] = load_as_f32<DT>(x, row_base + i0 + e);
+    }
+  }
 }
 
 __device__ __forceinline__ int bucketize(const float *bnd, int levels_pow2, float v) {
@@ -180,7 +245,7 @@ __device__ __forceinline__ void fwht_regs(float (&v)[N], int limit) {
 }
 
 // Lane exchanges for the butterflies between lanes l and l xor J: DPP quad permutes (1, 2),
-// masked row shifts (4), a row rotate (8); wavefront shuffles for 16 and 32.
+// masked row shifts (4), a row rotate (8); wavefront shuffles for 16 and 32 (see also swap_stage).
 __device__ __forceinline__ float dpp_xor1(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
 }
@@ -203,6 +268,29 @@ __device__ __forceinline__ float lane_xor(float v) {
   else if constexpr (J == 4) return dpp_xor4(v);
   else if constexpr (J == 8) return dpp_xor8(v);
   else return __shfl_xor(v, J, 64);
+}
+
+// Butterflies between lanes l and l xor J for J = 16, 32 without LDS traffic, two registers at a
+// time.  The swap instruction exchanges the upper half of each 2J-lane group of `a` with the
+// lower half of the same group of `b`; afterwards a holds the lower-half values of both
+// registers and b the upper-half values, lane for lane, so sum and difference are plain
+// register operations, and a second swap puts them back where the butterfly wants them
+// (lower lane: y + other, upper lane: other - y, the same two operands as with a lane exchange).
+template <int J>
+__device__ __forceinline__ void swap_stage(float (&y)[kChunk]) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  auto swap = [](float a, float b) -> u32x2 {
+    if constexpr (J == 16) return __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    else return __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  };
+#pragma unroll
+  for (int e = 0; e < kChunk; e += 2) {
+    const u32x2 r = swap(y[e], y[e + 1]);
+    const float lo = __uint_as_float(r.x), hi = __uint_as_float(r.y);
+    const u32x2 o = swap(lo + hi, lo - hi);
+    y[e] = __uint_as_float(o.x);
+    y[e + 1] = __uint_as_float(o.y);
+  }
 }
 
 // x / (s + eps) is evaluated as q0 = x*r, then two residual corrections
@@ -262,6 +350,10 @@ __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a)
   uint2 *cells = reinterpret_cast<uint2 *>(red + 4);            // kMaxCells x (boundary, count below)
   int *cells_bad = reinterpret_cast<int *>(cells + kMaxCells);  // 4 ints (one used)
   float *xbuf = reinterpret_cast<float *>(cells_bad + 4);       // Kp elements of Stage::kBytes
+  // The window of the input map sits behind everything else, so that no other LDS address depends on it.
+  const bool windowed = a.map != nullptr && a.map_lo >= 0;     // bf16 only (the launcher decides)
+  uint16_t *hot_lds = reinterpret_cast<uint16_t *>(smem + a.map_lds_offset);  // kHotBytes, only when windowed
+  const uint16_t *hot = windowed ? hot_lds : nullptr;
   uint16_t *xbuf16 = reinterpret_cast<uint16_t *>(xbuf);
   uint8_t *cbuf = reinterpret_cast<uint8_t *>(xbuf) + static_cast<size_t>(Kp) * Stage::kBytes;  // Kp bytes, big-block path only
   float *psum = reinterpret_cast<float *>(cbuf + (LOG_G > 0 ? Kp : 0));  // [passes][256], only with several pass groups
@@ -278,18 +370,30 @@ __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a)
     cent[i] = (a.cents != nullptr && i < a.levels) ? a.cents[i] : 0.0f;
   }
   if (tid == 0) cells_bad[0] = 0;
+  if (windowed) {  // both signs of the window, 16 bytes per thread and step; the rows are mapped before the first barrier below
+    for (int i = tid; i < kHotBytes / 16; i += nthreads) {
+      const int sign = i / (kHotHalf * 2 / 16), j = i % (kHotHalf * 2 / 16);
+      reinterpret_cast<uint4 *>(hot_lds)[i] = reinterpret_cast<const uint4 *>(a.map + (sign << 15) + a.map_lo)[j];
+    }
+    __syncthreads();
+  }
 
   // ---- phase A: stage the row, sum of squares in the documented order --------
   const int64_t row_base = row * K;
   float q = 0.0f;
-  for (int p = pg; p < a.passes; p += groups_n) {
-    const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
-    float f[kChunk];
-    if constexpr (Stage::k16) {
-      uint4 raw = make_uint4(0u, 0u, 0u, 0u);
-      if (i0 + kChunk <= K) raw = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(a.x) + row_base + i0);
-      *reinterpret_cast<uint4 *>(xbuf16 + i0) = raw;
-      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  auto square_sum = [&](const float (&f)[kChunk], int p) {
+    float s[kChunk];
+#pragma unroll
+    for (int e = 0; e < kChunk; ++e) s[e] = f[e] * f[e];
+    const float v8 = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+    if (groups_n == 1) q = (p == 0) ? v8 : q + v8;
+    else psum[p * kThreads + t] = v8;
+  };
+  if constexpr (Stage::k16) {
+    auto stage16 = [&](const uint4 rw, int p, int64_t i0) {
+      *reinterpret_cast<uint4 *>(xbuf16 + i0) = rw;
+      const uint32_t w[4] = {rw.x, rw.y, rw.z, rw.w};
+      float f[kChunk];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if constexpr (DT == OQ_BF16) {
@@ -300,18 +404,36 @@ __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a)
           f[2 * j + 1] = f16_bits_to_f32(static_cast<uint16_t>(w[j] >> 16));
         }
       }
+      square_sum(f, p);
+    };
+    const uint16_t *xrow = static_cast<const uint16_t *>(a.x) + row_base;
+    // Two loops on purpose: with the table lookup inside it, the compiler schedules the plain
+    // loop (and the passes after it) measurably worse.
+    if (a.map == nullptr) {
+      for (int p = pg; p < a.passes; p += groups_n) {
+        const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
+        uint4 rw = make_uint4(0u, 0u, 0u, 0u);
+        if (i0 + kChunk <= K) rw = *reinterpret_cast<const uint4 *>(xrow + i0);
+        stage16(rw, p, i0);
+      }
     } else {
-      load_chunk<DT, VEC>(a.x, row_base, i0, K, f);
+      for (int p = pg; p < a.passes; p += groups_n) {
+        const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
+        uint4 rw = make_uint4(0u, 0u, 0u, 0u);
+        if (i0 + kChunk <= K) rw = map_raw8<DT>(*reinterpret_cast<const uint4 *>(xrow + i0), a, hot);
+        stage16(rw, p, i0);
+      }
+    }
+  } else {
+    for (int p = pg; p < a.passes; p += groups_n) {
+      const int64_t i0 = static_cast<int64_t>(p) * kPass + t * kChunk;
+      float f[kChunk];
+      load_chunk<DT, VEC>(a, hot, row_base, i0, f);
       float4 *dst = reinterpret_cast<float4 *>(xbuf + i0);
       dst[0] = make_float4(f[0], f[1], f[2], f[3]);
       dst[1] = make_float4(f[4], f[5], f[6], f[7]);
+      square_sum(f, p);
     }
-    float s[kChunk];
-#pragma unroll
-    for (int e = 0; e < kChunk; ++e) s[e] = f[e] * f[e];
-    const float v8 = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
-    if (groups_n == 1) q = (p == 0) ? v8 : q + v8;
-    else psum[p * kThreads + t] = v8;
   }
   if (groups_n > 1) {  // the lane's passes were summed by different threads: add them left to right
     __syncthreads();
@@ -431,8 +553,13 @@ __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a)
       lane_stage(std::integral_constant<int, 2>{});
       lane_stage(std::integral_constant<int, 4>{});
       lane_stage(std::integral_constant<int, 8>{});
-      lane_stage(std::integral_constant<int, 16>{});
-      lane_stage(std::integral_constant<int, 32>{});
+      if constexpr (BIG) {  // LDS is the busier unit on this path, the ALUs on the other
+        swap_stage<16>(y);
+        swap_stage<32>(y);
+      } else {
+        lane_stage(std::integral_constant<int, 16>{});
+        lane_stage(std::integral_constant<int, 32>{});
+      }
       if constexpr (!BIG) {
         int code[kChunk];
 #pragma unroll
@@ -491,6 +618,12 @@ int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {  // sme
   const int pass_groups = (a.M <= 64 && a.passes >= 2 && getenv("OQ_RQ_ONE_GROUP") == nullptr) ? (a.passes >= 3 ? 4 : 2) : 1;
   dim3 grid(static_cast<unsigned>(a.M)), block(pass_groups > 1 ? kThreads * pass_groups : 64 * waves);
   if (pass_groups > 1) smem += static_cast<size_t>(a.passes) * kThreads * sizeof(float);
+  RqArgs args = a;
+  if (a.map_lo >= 0) {
+    smem = (smem + 15) & ~static_cast<size_t>(15);
+    args.map_lds_offset = static_cast<int>(smem);
+    smem += kHotBytes;
+  }
 #define OQ_RQ_CASE(LG)                                                                           \
   case LG: {                                                                                     \
     auto kern = rotate_quantize_kernel<DT, VEC, LG>;                                             \
@@ -500,7 +633,7 @@ int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {  // sme
                               static_cast<int>(smem)) != hipSuccess)                            \
         return fail(OQ_ERR_LAUNCH, "rotate_quantize: cannot reserve %zu bytes of LDS", smem);    \
     }                                                                                            \
-    hipLaunchKernelGGL(kern, grid, block, smem, stream, a);                                      \
+    hipLaunchKernelGGL(kern, grid, block, smem, stream, args);                                   \
     break;                                                                                       \
   }
   switch (log_g) {
@@ -523,7 +656,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              const int8_t *signs, const float *boundaries, const float *centroids,
                              int levels, int64_t block, float eps, float inv_sqrt_block,
                              void *codes_out, int code_format, void *values_out, int values_mode,
-                             float *norms_out, hipStream_t stream) {
+                             float *norms_out, const uint16_t *input_map, hipStream_t stream) {
   if (M < 0 || K <= 0) return fail(OQ_ERR_INVALID, "rotate_quantize: M=%lld K=%lld", (long long)M, (long long)K);
   if (M == 0) return OQ_OK;
   if (x == nullptr || perm == nullptr || signs == nullptr || boundaries == nullptr)
@@ -548,7 +681,18 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
       return fail(OQ_ERR_INVALID, "rotate_quantize: values_mode set but values_out/centroids is null");
   }
 
+  if (input_map != nullptr) {
+    if (x_dtype != OQ_F16 && x_dtype != OQ_BF16)
+      return fail(OQ_ERR_INVALID, "rotate_quantize: an input map needs 16-bit inputs (x_dtype %d)", x_dtype);
+    if ((reinterpret_cast<uintptr_t>(input_map) & 15u) != 0)
+      return fail(OQ_ERR_INVALID, "rotate_quantize: the input map must be 16-byte aligned");
+  }
+
   RqArgs a;
+  a.map = input_map;
+  // bf16: |x| in [2^-10, 2^6) is served from LDS (exponent field 117 .. 132)
+  a.map_lo = (input_map != nullptr && x_dtype == OQ_BF16) ? (117 << 7) : -1;
+  a.map_lds_offset = 0;
   a.x = x; a.M = M; a.K = K; a.perm = perm; a.signs = signs; a.bounds = boundaries;
   a.cents = centroids; a.levels = levels;
   a.levels_pow2 = 2;

@@ -35,13 +35,14 @@ _LIB.define(
     "quantized_linear(Tensor x, Tensor permutation, Tensor signs, Tensor act_centroids, "
     "Tensor act_boundaries, Tensor packed_weight_indices, Tensor row_norms, Tensor weight_centroids, "
     "Tensor? bias, int block_size, float eps, float inv_sqrt_block, int activation_bits, "
-    "int weight_bits, int out_features) -> Tensor"
+    "int weight_bits, int out_features, Tensor? input_map=None) -> Tensor"
 )
 
 
 def quantized_linear_forward(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
+    input_map=None,
 ):
     in_features = x.shape[-1]
     if bias is not None and bias.dtype != x.dtype:
@@ -49,7 +50,7 @@ def quantized_linear_forward(
     if activation_bits <= 4 and in_features % 2 == 0:
         codes, _, norms = ops.rotate_quantize(
             x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
-            inv_sqrt_block=inv_sqrt_block, code_format="nibble")
+            inv_sqrt_block=inv_sqrt_block, code_format="nibble", input_map=input_map)
         return ops.packed_linear(
             codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
             code_format="nibble", activation_bits=activation_bits, weight_bits=weight_bits,
@@ -59,14 +60,15 @@ def quantized_linear_forward(
         # wider activation codes: one code per byte into the all-table tile / streaming kernels
         codes, _, norms = ops.rotate_quantize(
             x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
-            inv_sqrt_block=inv_sqrt_block, code_format="u8")
+            inv_sqrt_block=inv_sqrt_block, code_format="u8", input_map=input_map)
         return ops.packed_linear(
             codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
             code_format="u8", activation_bits=activation_bits, weight_bits=weight_bits,
             out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
     _, unit, norms = ops.rotate_quantize(
         x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
-        inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16")
+        inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16",
+        input_map=input_map)
     return ops.matmul_packed_weight_values(
         unit, packed_weight_indices, row_norms, weight_centroids, bits=weight_bits,
         out_features=out_features, in_features=in_features, bias=bias,
@@ -76,6 +78,7 @@ def quantized_linear_forward(
 def _quantized_linear_fake(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
+    input_map=None,
 ):
     return x.new_empty((*x.shape[:-1], out_features))
 
@@ -125,6 +128,22 @@ class OrbitLinear(nn.Module):
         for name, tensor in self._constants().items():
             self.register_buffer(name, tensor.to(device), persistent=False)
         self.last_effective_runtime_mode: str | None = None
+        self._input_activation = None  # (fn, dtype) once fuse_input_activation() was called
+        self.register_buffer("_input_activation_table", None, persistent=False)
+
+    def fuse_input_activation(self, fn, *, dtype: torch.dtype = torch.bfloat16) -> "OrbitLinear":
+        """Make forward(x) return what forward(fn(x)) returns, bit for bit, without a separate
+        elementwise kernel and without fn(x) being written to memory: fn (elementwise, e.g. the
+        GELU between the two linears of an MLP) is handed to the quantize kernel as the table of
+        its values on all 65536 inputs of `dtype`, filled here by fn itself.  Inputs of another
+        dtype are refused.  `fn=None` undoes it."""
+        if fn is None:
+            self._input_activation = None
+            self._input_activation_table = None
+            return self
+        self._input_activation = (fn, dtype)
+        self._input_activation_table = ops.activation_table(fn, dtype, self.packed_weight_indices.device)
+        return self
 
     def _constants(self) -> dict[str, torch.Tensor]:
         return {
@@ -162,6 +181,9 @@ class OrbitLinear(nn.Module):
         device = self.packed_weight_indices.device
         for name, tensor in self._constants().items():
             setattr(self, name, tensor.to(device))
+        if self._input_activation is not None and device.type == "cuda":
+            # a dtype cast must not touch the table's bits: fill it again
+            self._input_activation_table = ops.activation_table(*self._input_activation, device)
         return result
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -172,13 +194,16 @@ class OrbitLinear(nn.Module):
                 "OrbitLinear runs on AMD GPUs only (torch device 'cuda'); there is no CPU fallback")
         if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
             raise ValueError("x must be float32, float16 or bfloat16")
+        table = self._input_activation_table
+        if table is not None and table.dtype != x.dtype:
+            raise ValueError(f"the fused input activation was built for {table.dtype}, got {x.dtype}")
         self.last_effective_runtime_mode = "hip_packed"
         return torch.ops.orbitquant_amd.quantized_linear(
             x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_centroids,
             self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
             self._weight_codebook_centroids, self.bias, self.rotation.block_size,
             self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
-            self.out_features)
+            self.out_features, table)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -67,8 +67,12 @@ def rotate_quantize(
     centroids: torch.Tensor | None = None,
     code_format: str | None = "u8",
     values: str | None = None,
+    input_map: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor | None, torch.Tensor | None, torch.Tensor]:
     """-> (codes or None, values or None, norms[...]).
+
+    input_map: None, or the table of an elementwise function f (`activation_table`): the
+    result is that of rotate_quantize(f(x)), bit for bit, without f(x) ever being stored.
 
     code_format: "u8" ([..., K] uint8), "nibble" ([..., K/2] uint8) or None.
     values: None, "scaled" (centroid*norm in x.dtype) or "unit_bf16" (bf16 centroid).
@@ -106,19 +110,40 @@ def rotate_quantize(
     if mode != OQ_VALUES_NONE and centroids is None:
         raise ValueError("centroids are required when values are requested")
     norms = torch.empty(m, dtype=torch.float32, device=x.device)
+    if input_map is not None:
+        if x.dtype not in (torch.float16, torch.bfloat16):
+            raise ValueError("an input map needs float16 or bfloat16 inputs")
+        if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device:
+            raise ValueError("input_map must hold 65536 entries of x's dtype on x's device")
+        input_map = input_map.contiguous()
     lib = _lib.load()
+    tail = (m, dim, permutation.data_ptr(), signs.data_ptr(), boundaries.data_ptr(), _ptr(centroids), levels,
+            int(block_size), float(eps), float(inv_sqrt_block), _ptr(codes), fmt, _ptr(out_values), mode,
+            norms.data_ptr(), _stream(x))
     with _OnDevice(x):
-        rc = lib.oq_rotate_quantize(
-            rows.data_ptr(), _dt(rows), m, dim, permutation.data_ptr(), signs.data_ptr(),
-            boundaries.data_ptr(), _ptr(centroids), levels, int(block_size), float(eps),
-            float(inv_sqrt_block), _ptr(codes), fmt, _ptr(out_values), mode, norms.data_ptr(),
-            _stream(x))
+        if input_map is None:
+            rc = lib.oq_rotate_quantize(rows.data_ptr(), _dt(rows), *tail)
+        else:
+            rc = lib.oq_rotate_quantize_mapped(rows.data_ptr(), _dt(rows), input_map.data_ptr(), *tail)
     _lib.check(rc, "oq_rotate_quantize")
     if codes is not None:
         codes = codes.reshape(*lead, codes.shape[-1])
     if out_values is not None:
         out_values = out_values.reshape(*lead, dim)
     return codes, out_values, norms.reshape(lead)
+
+
+def activation_table(fn, dtype: torch.dtype, device) -> torch.Tensor:
+    """The table of an elementwise function for `rotate_quantize(input_map=...)`: fn applied
+    to all 65536 values of a 16-bit dtype, in bit order, by the framework's own kernel for fn
+    on `device`, so the fused path returns exactly what fn followed by the quantizer returns."""
+    if dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("activation tables exist for float16 and bfloat16 only")
+    bits = torch.arange(65536, dtype=torch.int32, device=device).to(torch.int16)
+    out = fn(bits.view(dtype))
+    if out.dtype != dtype or out.shape != bits.shape:
+        raise ValueError("fn must be elementwise and keep the dtype")
+    return out.contiguous()
 
 
 def packed_linear(

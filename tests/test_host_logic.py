@@ -187,3 +187,22 @@ def test_dropin_package_surface_and_validation():
                                  out_features=1, in_features=16)
     with pytest.raises(RuntimeError):
         pkg.quantize_activations_packed_w4(x, torch.arange(16), torch.ones(16), torch.zeros(15), inv_sqrt_block=0.25)
+
+
+def test_activation_table_on_the_cpu():
+    """The table handed to the quantize kernel is the function itself on all 65536 bit patterns."""
+    from orbitquant_amd import ops
+
+    gelu = torch.nn.functional.gelu
+    for dtype in (torch.bfloat16, torch.float16):
+        table = ops.activation_table(gelu, dtype, "cpu")
+        assert table.dtype == dtype and table.shape == (65536,)
+        for value in (0.0, 1.0, -1.0, 0.37, -3.5, 100.0):
+            t = torch.tensor([value], dtype=dtype)
+            bits = int(t.view(torch.int16).item()) & 0xFFFF
+            assert torch.equal(table[bits : bits + 1], gelu(t))
+        assert torch.isnan(table[(torch.tensor([float("nan")], dtype=dtype).view(torch.int16).item()) & 0xFFFF])
+    with pytest.raises(ValueError):
+        ops.activation_table(gelu, torch.float32, "cpu")
+    with pytest.raises(ValueError):
+        ops.activation_table(lambda t: t.float(), torch.bfloat16, "cpu")
