@@ -142,6 +142,30 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                      void *stream);
 
 /*
+ * The whole quantized-linear forward in one call: oq_rotate_quantize (through
+ * `input_map` when it is not NULL, see oq_rotate_quantize_mapped) followed by
+ * oq_packed_linear, with the same results bit for bit.  It is the native form of the
+ * reference layer's forward (src/orbitquant/layers.py:1079-1455: quantize_activations_*
+ * then matmul_packed_*), which exists there only as Python glue between two ops.
+ *
+ * One token (M == 1) of a 16-bit dtype with a_bits <= 4 and w_bits 2, 3 or 4 is a SINGLE
+ * launch: every workgroup of the streaming kernel quantizes the token itself while its first
+ * weight loads are in flight, so decoding pays one launch per linear and the scratch buffers
+ * are not touched (they may be NULL).  Every other shape is the two launches, with the codes
+ * ([M, K/2] bytes when a_bits <= 4 and K is even, else [M, K]) and norms (fp32 [M]) passing
+ * through the caller's scratch buffers (16-byte aligned).
+ */
+int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
+                        int64_t M, int64_t K,
+                        const int32_t *perm, const int8_t *signs,
+                        const float *boundaries, const float *act_centroids, int a_bits,
+                        int64_t block, float eps, float inv_sqrt_block,
+                        const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                        const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
+                        void *codes_scratch, float *norms_scratch,
+                        void *out, int out_dtype, void *stream);
+
+/*
  * Packed-weight matmul on float activations:
  *
  *   out[m,n] = (sum_k x[m,k] * c_w[idx[n,k]]) * r_w[n] + bias[n]      (out in x's dtype)

@@ -34,6 +34,10 @@ SOURCES = {
     "packed_gemm_bytes.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
+    "token_linear.hip": [],
+    "token_linear_w2.hip": [],
+    "token_linear_w3.hip": [],
+    "token_linear_w4.hip": [],
 }
 
 

@@ -37,6 +37,13 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              int levels, int64_t block, float eps, float inv_sqrt_block,
                              void *codes_out, int code_format, void *values_out, int values_mode,
                              float *norms_out, const uint16_t *input_map, hipStream_t stream);
+bool token_linear_supported(int x_dtype, int64_t M, int64_t N, int64_t K, int levels, int bits, const void *x,
+                            const int32_t *perm, const int8_t *signs);
+int token_linear_dispatch(const void *x, int x_dtype, const uint16_t *input_map, int64_t K, const int32_t *perm,
+                          const int8_t *signs, const float *boundaries, const float *act_cents, int levels,
+                          int64_t block, float eps, float inv_sqrt_block, const uint8_t *packed_w, int bits,
+                          const uint16_t *row_norms, const float *w_cents, const void *bias, int bias_dtype,
+                          int64_t N, void *out, int out_dtype, hipStream_t stream, bool *launched);
 int generic_matmul_float(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
                          int bits, const uint16_t *row_norms, const float *w_cents, const void *bias,
                          int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
@@ -140,6 +147,36 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                          bias, bias_dtype, M, N, K, out, out_dtype, s);
   return generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
                               w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+}
+
+int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
+                        const int32_t *perm, const int8_t *signs, const float *boundaries,
+                        const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
+                        const uint8_t *packed_w, int w_bits, const uint16_t *row_norms, const float *w_centroids,
+                        const void *bias, int bias_dtype, int64_t N, void *codes_scratch, float *norms_scratch,
+                        void *out, int out_dtype, void *stream) {
+  if (int rc = check_matmul_common("quantized_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
+  if (M == 0) return OQ_OK;
+  if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "quantized_linear: a_bits=%d", a_bits);
+  if (act_centroids == nullptr) return fail(OQ_ERR_INVALID, "quantized_linear: null activation centroids");
+  const int levels = 1 << a_bits;
+  hipStream_t s = as_stream(stream);
+  if (aligned16(packed_w) && token_linear_supported(x_dtype, M, N, K, levels, w_bits, x, perm, signs)) {
+    bool launched = false;
+    const int rc = token_linear_dispatch(x, x_dtype, input_map, K, perm, signs, boundaries, act_centroids, levels, block,
+                                         eps, inv_sqrt_block, packed_w, w_bits, row_norms, w_centroids, bias,
+                                         bias_dtype, N, out, out_dtype, s, &launched);
+    if (rc != OQ_OK || launched) return rc;
+  }
+  if (codes_scratch == nullptr || norms_scratch == nullptr)
+    return fail(OQ_ERR_INVALID, "quantized_linear: this shape takes two launches and needs the scratch buffers");
+  const int fmt = (a_bits <= 4 && (K & 1) == 0) ? OQ_CODES_NIBBLE : OQ_CODES_U8;
+  if (int rc = rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, nullptr, levels, block, eps,
+                                        inv_sqrt_block, codes_scratch, fmt, nullptr, OQ_VALUES_NONE, norms_scratch,
+                                        input_map, s))
+    return rc;
+  return oq_packed_linear(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
+                          w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, stream);
 }
 
 int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,

@@ -1,185 +1,15 @@
-// Small-M (decode-sized, M <= 16) packed-weight linear: a pure stream over the
-// packed index bytes.
-//
-// The token rows are the 16-row side of v_mfma_f32_16x16x32_bf16 (rows beyond M
-// are padding), sixteen weight rows are the other side, so the k-reduction
-// happens inside the matrix core and the weights are streamed from HBM exactly
-// once whatever M is.  A workgroup owns 16*R consecutive weight rows for the
-// whole K range; its wavefronts split K between them and add their partial
-// tiles through LDS in a fixed order (wave 0, 1, 2, ...), so results do not
-// depend on timing.
-//
-// K is cut like in the tiled GEMM: in a K-step of 128, lane group g (0..3) owns
-// the contiguous run k0+32g .. k0+32g+31 of its row and MFMA q (0..3) consumes
-// values 8q..8q+7 of every run.
-//
-// Lookup tables: the 64 KB block of 256-byte rows the tiled GEMM uses (weight
-// entry e 32 times in bytes 0..127 of row e, activation entry e in bytes
-// 128..255; lane l reads copy l%32, a byte-indexed lookup is one v_perm_b32 plus
-// one ds_read_b32).  The packed stream is requested first thing; the tables are
-// built meanwhile from centroids fetched with SCALAR loads, which do not queue
-// behind the vector loads of the stream, and spread over the lanes so that every lane can pick the two values of its table entry with
-// wavefront shuffles.  After the main loop the same LDS holds the partial sums.
-#include <stdio.h>
-#include <stdlib.h>
-
-#include "packed_decode.h"
+// Small-M (decode-sized, M <= 16) packed-weight linear on activation codes: kernel, launch
+// configuration and argument checks.  The arithmetic is in packed_gemv_body.h.
+#include "packed_gemv_body.h"
 
 namespace oq {
 namespace {
 
-struct GemvArgs {
-  const uint8_t *a;          // activation codes: [M, K/2] two per byte, or [M, K] one per byte
-  const float *row_scale;    // [M] or NULL
-  const float *act_cents;
-  int a_levels;
-  const uint8_t *w;
-  const uint16_t *row_norms;
-  const float *w_cents;
-  const void *bias;
-  int bias_dtype;
-  int M;
-  int64_t N, K;
-  void *out;
-  int out_dtype;
-};
+using namespace gemv;
 
-constexpr int kDepth = 1;  // K-steps of 128 fetched per batch of global loads (two batches in flight: decode of one overlaps the stream of the next)
-constexpr int kGemvTableBytes = kRowTableBytes;
-
-// BYTES: activation codes come one per byte (widths above 4 bits) instead of two per byte.
 template <bool BYTES, int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
-  constexpr int kAVec = BYTES ? 2 : 1;      // 16-byte loads of activation codes per lane and K-step
-  constexpr int kAStep = 64 * kAVec;        // bytes of one activation row per K-step of 128
-  static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
-  __shared__ __attribute__((aligned(65536))) uint32_t lds[kGemvTableBytes / 4];
-  float *partial = reinterpret_cast<float *>(lds);  // [WAVES][R][64][4], after the main loop
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, grp = lane >> 4;
-  const uint32_t lds_base = lds_byte_address(lds);  // a multiple of 65536 by the alignment
-  const uint32_t w_off = lds_base + 4 * (lane & 31), a_off = lds_base + 128 + 4 * (lane & 31);
-  const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * R);
-
-  const int steps = static_cast<int>(g.K / 128);
-  const int s_begin = static_cast<int>(static_cast<int64_t>(steps) * wave / WAVES);
-  const int s_end = static_cast<int>(static_cast<int64_t>(steps) * (wave + 1) / WAVES);
-
-  const int64_t w_row_bytes = g.K * BITS / 8;
-  const uint8_t *ap = g.a + static_cast<int64_t>(min(r, g.M - 1)) * (BYTES ? g.K : g.K / 2) + grp * (16 * kAVec);
-  const uint8_t *wp[R];
-#pragma unroll
-  for (int j = 0; j < R; ++j) {
-    const int64_t row = min(n_base + 16 * j + r, g.N - 1);
-    wp[j] = g.w + row * w_row_bytes + grp * (4 * BITS);
-  }
-
-  // a batch = kDepth K-steps: every load of the batch is issued before anything waits on it
-  struct Batch {
-    uint4 a[kDepth][kAVec];
-    uint32_t w[kDepth][R][BITS];
-  };
-  auto fetch = [&](int s0, Batch &bt) {
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-      const int s = min(s0 + d, s_end - 1);  // clamped: stays inside the row, result unused
-#pragma unroll
-      for (int v = 0; v < kAVec; ++v)
-        bt.a[d][v] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * kAStep + 16 * v);
-#pragma unroll
-      for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s) * (16 * BITS), bt.w[d][j]);
-    }
-  };
-
-  f32x4 acc[R];
-#pragma unroll
-  for (int j = 0; j < R; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  auto consume = [&](int s0, const Batch &bt) {
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-      if (s0 + d < s_end) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          uint4 af;
-          if constexpr (!BYTES) {
-            const uint4 v = bt.a[d][0];
-            af = decode_bytes(q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w, a_off);
-          } else {  // eight single-code lookups (value in both halves), merged two by two
-            const uint4 v = bt.a[d][q >> 1];
-            const uint4 e0 = decode_bytes((q & 1) ? v.z : v.x, a_off), e1 = decode_bytes((q & 1) ? v.w : v.y, a_off);
-            af = make_uint4(__builtin_amdgcn_perm(e0.y, e0.x, 0x07060100u), __builtin_amdgcn_perm(e0.w, e0.z, 0x07060100u),
-                            __builtin_amdgcn_perm(e1.y, e1.x, 0x07060100u), __builtin_amdgcn_perm(e1.w, e1.z, 0x07060100u));
-          }
-#pragma unroll
-          for (int j = 0; j < R; ++j) {
-            uint4 bf;
-            if constexpr (BITS == 4) bf = decode_bytes(bt.w[d][j][q], w_off);
-            else bf = decode_w<BITS, 6>(bt.w[d][j], q, w_off);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
-                                                             __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
-          }
-        }
-      }
-    }
-  };
-
-  // ---- the packed stream first ------------------------------------------------------
-  Batch b0, b1;
-  if (s_begin < s_end) fetch(s_begin, b0);
-  if (s_begin + kDepth < s_end) fetch(s_begin + kDepth, b1);
-
-  // epilogue operands of the item this thread will finish (item = tid when tid < 64*R)
-  const int ep_j = tid >> 6, ep_l = tid & 63;
-  const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
-  float ep_rn = 0.0f, ep_bv = 0.0f, ep_sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-  if (tid < 64 * R && ep_n < g.N) {
-    ep_rn = bf16_bits_to_f32(g.row_norms[ep_n]);
-    if (g.bias != nullptr) ep_bv = load_dyn_f32(g.bias, g.bias_dtype, ep_n);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int m = 4 * (ep_l >> 4) + e;
-      if (g.row_scale != nullptr && m < g.M) ep_sc[e] = g.row_scale[m];
-    }
-  }
-
-  // ---- tables (built while the stream is in flight) ---------------------------------------
-  build_row_tables<BITS, WAVES, BYTES>(lds, g.w_cents, g.act_cents, g.a_levels);
-  __syncthreads();
-
-  for (int s = s_begin; s < s_end; s += 2 * kDepth) {
-    consume(s, b0);
-    if (s + 2 * kDepth < s_end) fetch(s + 2 * kDepth, b0);
-    if (s + kDepth < s_end) consume(s + kDepth, b1);
-    if (s + 3 * kDepth < s_end) fetch(s + 3 * kDepth, b1);
-  }
-
-  // ---- cross-wave sum in LDS (the tables are dead), fixed order ------------------------
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < R; ++j)
-    *reinterpret_cast<float4 *>(partial + ((wave * R + j) * 64 + lane) * 4) =
-        make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
-  __syncthreads();
-  // accumulator e of lane l: token row 4*(l/16) + e, weight row l%16
-  if (tid < 64 * R && ep_n < g.N) {
-    float4 sum = *reinterpret_cast<const float4 *>(partial + ((0 * R + ep_j) * 64 + ep_l) * 4);
-    for (int w = 1; w < WAVES; ++w) {
-      const float4 p = *reinterpret_cast<const float4 *>(partial + ((w * R + ep_j) * 64 + ep_l) * 4);
-      sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
-    }
-    const float v[4] = {sum.x, sum.y, sum.z, sum.w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int m = 4 * (ep_l >> 4) + e;
-      if (m >= g.M) continue;
-      const float y = v[e] * ep_sc[e] * ep_rn + ep_bv;
-      const int64_t o = static_cast<int64_t>(m) * g.N + ep_n;
-      if (g.out_dtype == OQ_BF16) static_cast<uint16_t *>(g.out)[o] = f32_to_bf16_bits(y);
-      else if (g.out_dtype == OQ_F16) static_cast<uint16_t *>(g.out)[o] = f32_to_f16_bits(y);
-      else static_cast<float *>(g.out)[o] = y;
-    }
-  }
+  packed_gemv_body<BYTES, BITS, R, WAVES, false>(g, [](auto) {});
 }
 
 template <bool BYTES, int BITS, int R, int WAVES>

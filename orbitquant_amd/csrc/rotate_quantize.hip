@@ -10,25 +10,19 @@ using namespace rq;
 template <int DT, bool VEC, int LOG_G>
 __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  rotate_quantize_row<DT, VEC, LOG_G>(a, smem, blockIdx.x, threadIdx.x, blockDim.x);
+  rotate_quantize_row<DT, VEC, LOG_G>(a, smem, blockIdx.x, threadIdx.x, blockDim.x, [] {});
 }
 
 template <int DT, bool VEC>
-int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {  // smem: bytes without the pass-group scratch
-  int log_g = 0;
-  for (int g = a.block / kLaneSpan; g > 1; g >>= 1) ++log_g;
+int launch_for_block(const RqArgs &a, hipStream_t stream) {
+  const int log_g = log2_groups(a);
   // a wavefront owns 512 consecutive elements of a pass: launch only the wavefronts a single-pass row needs
   const int waves = a.K >= 3 * kLaneSpan ? 4 : static_cast<int>((a.K + kLaneSpan - 1) / kLaneSpan);
   // few rows (decode): the chip is empty anyway, so run the passes of a long row side by side
   const int pass_groups = (a.M <= 64 && a.passes >= 2 && getenv("OQ_RQ_ONE_GROUP") == nullptr) ? (a.passes >= 3 ? 4 : 2) : 1;
   dim3 grid(static_cast<unsigned>(a.M)), block(pass_groups > 1 ? kThreads * pass_groups : 64 * waves);
-  if (pass_groups > 1) smem += static_cast<size_t>(a.passes) * kThreads * sizeof(float);
   RqArgs args = a;
-  if (a.map_lo >= 0) {
-    smem = (smem + 15) & ~static_cast<size_t>(15);
-    args.map_lds_offset = static_cast<int>(smem);
-    smem += kHotBytes;
-  }
+  const size_t smem = lds_bytes(args, DT, VEC, pass_groups);
 #define OQ_RQ_CASE(LG)                                                                           \
   case LG: {                                                                                     \
     auto kern = rotate_quantize_kernel<DT, VEC, LG>;                                             \
@@ -57,13 +51,19 @@ int launch_for_block(const RqArgs &a, size_t smem, hipStream_t stream) {  // sme
 
 }  // namespace
 
-int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
-                             const int8_t *signs, const float *boundaries, const float *centroids,
-                             int levels, int64_t block, float eps, float inv_sqrt_block,
-                             void *codes_out, int code_format, void *values_out, int values_mode,
-                             float *norms_out, const uint16_t *input_map, hipStream_t stream) {
+int rotate_quantize_prepare(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
+                            const int8_t *signs, const float *boundaries, const float *centroids,
+                            int levels, int64_t block, float eps, float inv_sqrt_block,
+                            void *codes_out, int code_format, void *values_out, int values_mode,
+                            float *norms_out, const uint16_t *input_map, rq::RqArgs *out, bool *vec_out) {
   if (M < 0 || K <= 0) return fail(OQ_ERR_INVALID, "rotate_quantize: M=%lld K=%lld", (long long)M, (long long)K);
-  if (M == 0) return OQ_OK;
+  if (x_dtype != OQ_F32 && x_dtype != OQ_F16 && x_dtype != OQ_BF16)
+    return fail(OQ_ERR_INVALID, "rotate_quantize: unknown x_dtype %d", x_dtype);
+  if (M == 0) {  // nothing to do, nothing to check
+    *out = rq::RqArgs{};
+    *vec_out = false;
+    return OQ_OK;
+  }
   if (x == nullptr || perm == nullptr || signs == nullptr || boundaries == nullptr)
     return fail(OQ_ERR_INVALID, "rotate_quantize: null input pointer");
   if (levels < 2 || levels > 256) return fail(OQ_ERR_INVALID, "rotate_quantize: levels=%d not in [2, 256]", levels);
@@ -109,20 +109,29 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
   a.values = values_mode == OQ_VALUES_NONE ? nullptr : values_out; a.values_mode = values_mode;
   a.norms = norms_out;
 
-  const size_t kp = static_cast<size_t>(a.passes) * kPass;
-  const bool big = block > kLaneSpan;
-
   auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-  const bool vec = (K % 8 == 0) && aligned16(x) && aligned16(perm) && aligned16(signs) &&
-                   (codes_out == nullptr || aligned16(codes_out)) &&
-                   (values_out == nullptr || aligned16(values_out));
-  const bool stage16 = vec && x_dtype != OQ_F32 && !big;  // RqStage::k16
-  const size_t smem = (256 + 256 + 4) * sizeof(float) + kMaxCells * 8 + 16 + kp * (stage16 ? 2 : 4) + (big ? kp : 0);
+  *vec_out = (K % 8 == 0) && aligned16(x) && aligned16(perm) && aligned16(signs) &&
+             (codes_out == nullptr || aligned16(codes_out)) &&
+             (values_out == nullptr || aligned16(values_out));
+  *out = a;
+  return OQ_OK;
+}
+
+int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
+                             const int8_t *signs, const float *boundaries, const float *centroids,
+                             int levels, int64_t block, float eps, float inv_sqrt_block,
+                             void *codes_out, int code_format, void *values_out, int values_mode,
+                             float *norms_out, const uint16_t *input_map, hipStream_t stream) {
+  RqArgs a;
+  bool vec = false;
+  const int rc = rotate_quantize_prepare(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
+                                         inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
+                                         input_map, &a, &vec);
+  if (rc != OQ_OK || M == 0) return rc;
   switch (x_dtype) {
-    case OQ_F32: return vec ? launch_for_block<OQ_F32, true>(a, smem, stream) : launch_for_block<OQ_F32, false>(a, smem, stream);
-    case OQ_F16: return vec ? launch_for_block<OQ_F16, true>(a, smem, stream) : launch_for_block<OQ_F16, false>(a, smem, stream);
-    case OQ_BF16: return vec ? launch_for_block<OQ_BF16, true>(a, smem, stream) : launch_for_block<OQ_BF16, false>(a, smem, stream);
-    default: return fail(OQ_ERR_INVALID, "rotate_quantize: unknown x_dtype %d", x_dtype);
+    case OQ_F32: return vec ? launch_for_block<OQ_F32, true>(a, stream) : launch_for_block<OQ_F32, false>(a, stream);
+    case OQ_F16: return vec ? launch_for_block<OQ_F16, true>(a, stream) : launch_for_block<OQ_F16, false>(a, stream);
+    default: return vec ? launch_for_block<OQ_BF16, true>(a, stream) : launch_for_block<OQ_BF16, false>(a, stream);
   }
 }
 

@@ -337,9 +337,12 @@ __device__ __forceinline__ void load_perm_signs(const RqArgs &a, int64_t c0, Per
 // thread's index in a workgroup of `block_threads` threads (64 * wavefronts, or 256 * pass
 // groups), all of which must make this call.  Codes, values and the norm go where `a` points
 // for row `row` (any address space reachable through a generic pointer).
-template <int DT, bool VEC, int LOG_G>
+// `after_loads()` is called once by every thread, as soon as its first pass has gathered its
+// inputs: from there on the only global loads it still waits for are the permutation / sign
+// prefetches of later passes (rows longer than one pass per thread).
+template <int DT, bool VEC, int LOG_G, typename AfterLoads>
 __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned char *smem, const int64_t row,
-                                                    const int tid, const int block_threads) {
+                                                    const int tid, const int block_threads, AfterLoads after_loads) {
   using Stage = RqStage<DT, VEC, LOG_G>;
   // Thread = (virtual lane t of the 256-lane pass structure, pass group pg).  With one group a
   // thread walks all passes of its lane; when few rows are in flight the launcher starts up to
@@ -545,7 +548,10 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
           else y[e] = 0.0f;
         }
       }
-      if constexpr (VEC) ps_cur = ps_nxt;
+      if constexpr (VEC) {
+        if (p + groups_n < a.passes) ps_cur = ps_nxt;  // same condition as the load: no wait where nothing was requested
+      }
+      if (pi == 0) after_loads();  // this thread's first permutation and signs have arrived and are used up
       fwht_regs<kChunk>(y, h);
       auto lane_stage = [&](auto jt) {
         constexpr int J = decltype(jt)::value;
@@ -576,6 +582,8 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) keep[pi][e] = y[e];
       }
+    } else if (pi == 0) {
+      after_loads();
     }
   }
 
@@ -615,5 +623,39 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
   }
 }
 
+
+// Host side: bytes of scratch rotate_quantize_row needs for a workgroup of `pass_groups`
+// groups of 256 threads (1: a single group, possibly of fewer wavefronts); sets the offset
+// of the input-map window in `a` when there is one.
+inline size_t lds_bytes(RqArgs &a, int x_dtype, bool vec, int pass_groups) {
+  const size_t kp = static_cast<size_t>(a.passes) * kPass;
+  const bool big = a.block > kLaneSpan;
+  const bool stage16 = vec && x_dtype != OQ_F32 && !big;  // RqStage::k16
+  size_t bytes = (256 + 256 + 4) * sizeof(float) + kMaxCells * 8 + 16 + kp * (stage16 ? 2 : 4) + (big ? kp : 0);
+  if (pass_groups > 1) bytes += static_cast<size_t>(a.passes) * kThreads * sizeof(float);
+  bytes = (bytes + 15) & ~static_cast<size_t>(15);
+  if (a.map_lo >= 0) {
+    a.map_lds_offset = static_cast<int>(bytes);
+    bytes += kHotBytes;
+  }
+  return bytes;
+}
+
+inline int log2_groups(const RqArgs &a) {  // the LOG_G template argument for a block size
+  int log_g = 0;
+  for (int g = a.block / kLaneSpan; g > 1; g >>= 1) ++log_g;
+  return log_g;
+}
+
 }  // namespace rq
+
+// Checks the arguments of oq_rotate_quantize and fills `out`; `vec` tells whether every
+// pointer and K allow the 16-byte access paths (the VEC template argument).  Returns OQ_OK,
+// or the status to hand back (the message is set).  Defined in rotate_quantize.hip.
+int rotate_quantize_prepare(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
+                            const int8_t *signs, const float *boundaries, const float *centroids,
+                            int levels, int64_t block, float eps, float inv_sqrt_block,
+                            void *codes_out, int code_format, void *values_out, int values_mode,
+                            float *norms_out, const uint16_t *input_map, rq::RqArgs *out, bool *vec);
+
 }  // namespace oq

@@ -11,11 +11,14 @@ implementation, so `torch.compile(fullgraph=True)` traces through it the way
 the reference's `orbitquant::packed_linear_forward` does (layers.py:38-72,
 1072-1077).  The op is stateless: every tensor it needs is an argument.
 
-Inside the op (the reference's `_forward_impl`, layers.py:1079-1455, for AMD):
+Inside the op (the reference's `_forward_impl`, layers.py:1079-1455, for AMD), one
+native call (`oq_quantized_linear`):
   1. fused rotate + per-token quantize (HIP) -> activation codes + token norms
   2. packed-weight matmul (HIP): streaming kernel for <= 16 tokens, MFMA tile
-     kernel otherwise; activation widths above 4 bits hand the matmul bf16
-     centroid values instead of nibble codes.
+     kernel otherwise.
+For a single token both run in ONE launch.  Shapes the code kernels do not take
+(activation widths above 4 bits with K not a multiple of 64 / 128) hand the matmul
+bf16 centroid values instead of codes.
 There is no dequantized-weight or CPU fallback on this path.
 """
 
@@ -47,24 +50,15 @@ def quantized_linear_forward(
     in_features = x.shape[-1]
     if bias is not None and bias.dtype != x.dtype:
         bias = bias.to(x.dtype)
-    if activation_bits <= 4 and in_features % 2 == 0:
-        codes, _, norms = ops.rotate_quantize(
-            x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
-            inv_sqrt_block=inv_sqrt_block, code_format="nibble", input_map=input_map)
-        return ops.packed_linear(
-            codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
-            code_format="nibble", activation_bits=activation_bits, weight_bits=weight_bits,
-            out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
     tokens = x.numel() // in_features
-    if (tokens > 16 and in_features % 64 == 0) or in_features % 128 == 0:
-        # wider activation codes: one code per byte into the all-table tile / streaming kernels
-        codes, _, norms = ops.rotate_quantize(
-            x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
-            inv_sqrt_block=inv_sqrt_block, code_format="u8", input_map=input_map)
-        return ops.packed_linear(
-            codes, norms, act_centroids, packed_weight_indices, row_norms, weight_centroids,
-            code_format="u8", activation_bits=activation_bits, weight_bits=weight_bits,
-            out_features=out_features, in_features=in_features, bias=bias, output_dtype=x.dtype)
+    if (activation_bits <= 4 and in_features % 2 == 0) or (tokens > 16 and in_features % 64 == 0) or in_features % 128 == 0:
+        # activation codes (two per byte up to 4 bits, else one per byte) into the tile / streaming
+        # kernels; one native call: a single launch for one token, two launches otherwise
+        return ops.quantized_linear(
+            x, permutation, signs, act_boundaries, act_centroids, packed_weight_indices, row_norms,
+            weight_centroids, block_size=block_size, eps=eps, inv_sqrt_block=inv_sqrt_block,
+            activation_bits=activation_bits, weight_bits=weight_bits, out_features=out_features, bias=bias,
+            input_map=input_map)
     _, unit, norms = ops.rotate_quantize(
         x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
         inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16",

@@ -191,6 +191,64 @@ def packed_linear(
     return out.reshape(*lead, out_features)
 
 
+def quantized_linear(
+    x: torch.Tensor,
+    permutation: torch.Tensor,
+    signs: torch.Tensor,
+    boundaries: torch.Tensor,
+    act_centroids: torch.Tensor,
+    packed_weight: torch.Tensor,
+    row_norms: torch.Tensor,
+    weight_centroids: torch.Tensor,
+    *,
+    block_size: int,
+    eps: float,
+    inv_sqrt_block: float,
+    activation_bits: int,
+    weight_bits: int,
+    out_features: int,
+    bias: torch.Tensor | None = None,
+    input_map: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """rotate_quantize followed by packed_linear in one native call (same results): a single
+    launch for one token of a 16-bit dtype (decode), two launches through scratch otherwise."""
+    _require_gpu(x, "x")
+    dim = x.shape[-1]
+    rows = x.contiguous().reshape(-1, dim)
+    m = rows.shape[0]
+    if permutation.dtype != torch.int32 or signs.dtype != torch.int8:
+        raise ValueError("permutation must be int32 and signs int8")
+    if boundaries.dtype != torch.float32 or act_centroids.dtype != torch.float32 or weight_centroids.dtype != torch.float32:
+        raise ValueError("boundaries and centroids must be float32")
+    if boundaries.numel() + 1 != 1 << activation_bits:
+        raise ValueError("boundaries do not match activation_bits")
+    if row_norms.dtype != torch.bfloat16 or packed_weight.dtype != torch.uint8:
+        raise ValueError("row_norms must be bfloat16 and packed_weight uint8")
+    expected = (out_features * dim * weight_bits + 7) // 8
+    if packed_weight.numel() != expected or row_norms.numel() != out_features:
+        raise ValueError(f"packed_weight must hold {expected} bytes and row_norms {out_features} values")
+    if input_map is not None:
+        if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device or x.dtype == torch.float32:
+            raise ValueError("input_map must hold 65536 entries of x's 16-bit dtype on x's device")
+        input_map = input_map.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+    nibble = activation_bits <= 4 and dim % 2 == 0
+    codes = torch.empty((m, dim // 2 if nibble else dim), dtype=torch.uint8, device=x.device)
+    norms = torch.empty(m, dtype=torch.float32, device=x.device)
+    out = torch.empty((m, out_features), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    with _OnDevice(x):
+        rc = lib.oq_quantized_linear(
+            rows.data_ptr(), _dt(rows), _ptr(input_map), m, dim, permutation.data_ptr(), signs.data_ptr(),
+            boundaries.data_ptr(), act_centroids.data_ptr(), int(activation_bits), int(block_size), float(eps),
+            float(inv_sqrt_block), packed_weight.data_ptr(), int(weight_bits), row_norms.data_ptr(),
+            weight_centroids.data_ptr(), _ptr(bias), _dt(bias) if bias is not None else 0, out_features,
+            codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _stream(x))
+    _lib.check(rc, "oq_quantized_linear")
+    return out.reshape(*x.shape[:-1], out_features)
+
+
 def matmul_packed_weight_values(
     x: torch.Tensor,
     packed_weight_indices: torch.Tensor,
