@@ -7,10 +7,10 @@ namespace {
 
 using namespace rq;
 
-template <int DT, bool VEC, int LOG_G>
+template <int DT, bool VEC, int LOG_G, bool FEW>
 __global__ __launch_bounds__(4 * kThreads) void rotate_quantize_kernel(RqArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  rotate_quantize_row<DT, VEC, LOG_G>(a, smem, blockIdx.x, threadIdx.x, blockDim.x, [] {});
+  rotate_quantize_row<DT, VEC, LOG_G, FEW>(a, smem, blockIdx.x, threadIdx.x, blockDim.x, [] {});
 }
 
 template <int DT, bool VEC>
@@ -23,9 +23,11 @@ int launch_for_block(const RqArgs &a, hipStream_t stream) {
   dim3 grid(static_cast<unsigned>(a.M)), block(pass_groups > 1 ? kThreads * pass_groups : 64 * waves);
   RqArgs args = a;
   const size_t smem = lds_bytes(args, DT, VEC, pass_groups);
-#define OQ_RQ_CASE(LG)                                                                           \
-  case LG: {                                                                                     \
-    auto kern = rotate_quantize_kernel<DT, VEC, LG>;                                             \
+  // the decode-sized variant exists for the 16-byte access paths only
+  const bool few = VEC && a.M <= 16;
+#define OQ_RQ_LAUNCH(KERN)                                                                       \
+  {                                                                                              \
+    auto kern = KERN;                                                                            \
     if (smem > 48 * 1024) {                                                                      \
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                              \
                               hipFuncAttributeMaxDynamicSharedMemorySize,                        \
@@ -33,8 +35,17 @@ int launch_for_block(const RqArgs &a, hipStream_t stream) {
         return fail(OQ_ERR_LAUNCH, "rotate_quantize: cannot reserve %zu bytes of LDS", smem);    \
     }                                                                                            \
     hipLaunchKernelGGL(kern, grid, block, smem, stream, args);                                   \
-    break;                                                                                       \
   }
+#define OQ_RQ_CASE(LG)                                                                           \
+  case LG:                                                                                       \
+    if constexpr (VEC) {                                                                         \
+      if (few) {                                                                                 \
+        OQ_RQ_LAUNCH((rotate_quantize_kernel<DT, VEC, LG, true>))                                \
+        break;                                                                                   \
+      }                                                                                          \
+    }                                                                                            \
+    OQ_RQ_LAUNCH((rotate_quantize_kernel<DT, VEC, LG, false>))                                   \
+    break;
   switch (log_g) {
     OQ_RQ_CASE(0)
     OQ_RQ_CASE(1)
@@ -46,6 +57,7 @@ int launch_for_block(const RqArgs &a, hipStream_t stream) {
       return fail(OQ_ERR_UNSUPPORTED, "rotate_quantize: block %d is larger than 16384", a.block);
   }
 #undef OQ_RQ_CASE
+#undef OQ_RQ_LAUNCH
   return check_launch("rotate_quantize");
 }
 

@@ -161,6 +161,22 @@ __device__ __forceinline__ int bucketize(const float *bnd, int levels_pow2, floa
   return code;
 }
 
+// The same search for N values at once: the N reads of a step are independent, so their LDS
+// latencies overlap (a thread of a decode-sized launch has nothing else to hide them behind).
+template <int N>
+__device__ __forceinline__ void bucketize_many(const float *bnd, int levels_pow2, const float (&v)[N], int (&code)[N]) {
+#pragma unroll
+  for (int e = 0; e < N; ++e) code[e] = 0;
+  for (int step = levels_pow2 >> 1; step > 0; step >>= 1) {
+    float b[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) b[e] = bnd[code[e] + step - 1];
+#pragma unroll
+    for (int e = 0; e < N; ++e)
+      if (b[e] < v[e]) code[e] += step;
+  }
+}
+
 // Faster bucketize for small codebooks: the interval [first boundary, last boundary] is cut
 // into kCells(levels) uniform cells; cell c stores how many boundaries lie in lower cells and
 // the one boundary inside it (+inf if none), so a value costs one LDS read and one compare:
@@ -340,7 +356,10 @@ __device__ __forceinline__ void load_perm_signs(const RqArgs &a, int64_t c0, Per
 // `after_loads()` is called once by every thread, as soon as its first pass has gathered its
 // inputs: from there on the only global loads it still waits for are the permutation / sign
 // prefetches of later passes (rows longer than one pass per thread).
-template <int DT, bool VEC, int LOG_G, typename AfterLoads>
+// FEW: the launch has a handful of rows (decode).  Then building the cell table (a barrier and
+// a microsecond of dependent LDS reads per workgroup) costs more than it saves, and the values
+// of a thread are searched together instead.  Same codes either way.
+template <int DT, bool VEC, int LOG_G, bool FEW, typename AfterLoads>
 __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned char *smem, const int64_t row,
                                                     const int tid, const int block_threads, AfterLoads after_loads) {
   using Stage = RqStage<DT, VEC, LOG_G>;
@@ -470,7 +489,7 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
 
   // ---- bucketize table (the boundaries are in LDS since the barrier above) ----------------
   CellMap cmap;
-  cmap.cells = a.levels <= 64 && a.levels >= 3 ? 8 * a.levels_pow2 : 0;
+  cmap.cells = !FEW && a.levels <= 64 && a.levels >= 3 ? 8 * a.levels_pow2 : 0;
   {
     const float lo = bnd[0], hi = bnd[a.levels - 2];
     cmap.scale = static_cast<float>(cmap.cells) / (hi - lo);
@@ -576,7 +595,15 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
       if constexpr (!BIG) {
         int code[kChunk];
 #pragma unroll
-        for (int e = 0; e < kChunk; ++e) code[e] = code_of(y[e] * a.inv_sqrt_block);
+        for (int e = 0; e < kChunk; ++e) {
+          if constexpr (!FEW) code[e] = code_of(y[e] * a.inv_sqrt_block);
+        }
+        if constexpr (FEW) {
+          float sv[kChunk];
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) sv[e] = y[e] * a.inv_sqrt_block;
+          bucketize_many<kChunk>(bnd, a.levels_pow2, sv, code);
+        }
         if (c0 < K) emit8<DT, VEC>(a, row, c0, code, cent, s_norm);
       } else {
 #pragma unroll
@@ -608,9 +635,19 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
 #pragma unroll
       for (int v = 0; v < G; ++v) z[v] = xbuf[base + kLaneSpan * v];
       fwht_regs<G>(z, G);
+      if constexpr (FEW) {
+        float sv[G];
+        int cd[G];
 #pragma unroll
-      for (int v = 0; v < G; ++v)
-        cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(code_of(z[v] * a.inv_sqrt_block));
+        for (int v = 0; v < G; ++v) sv[v] = z[v] * a.inv_sqrt_block;
+        bucketize_many<G>(bnd, a.levels_pow2, sv, cd);
+#pragma unroll
+        for (int v = 0; v < G; ++v) cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(cd[v]);
+      } else {
+#pragma unroll
+        for (int v = 0; v < G; ++v)
+          cbuf[base + kLaneSpan * v] = static_cast<uint8_t>(code_of(z[v] * a.inv_sqrt_block));
+      }
     }
     __syncthreads();
     for (int64_t c0 = static_cast<int64_t>(tid) * kChunk; c0 < K; c0 += static_cast<int64_t>(max(nthreads, kThreads)) * kChunk) {

@@ -29,7 +29,7 @@ __global__ __launch_bounds__(64 * kTokenWaves) void token_linear_kernel(rq::RqAr
   g.row_scale = norm;
   const int tid = threadIdx.x;
   gemv::packed_gemv_body<false, BITS, R, kTokenWaves, true>(g, [&](auto issue_weights) {
-    rq::rotate_quantize_row<DT, true, LOG_G>(q, smem, 0, tid, 64 * kTokenWaves, issue_weights);
+    rq::rotate_quantize_row<DT, true, LOG_G, true>(q, smem, 0, tid, 64 * kTokenWaves, issue_weights);
   });
 }
 
