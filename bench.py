@@ -464,6 +464,36 @@ def bench_c5(args, device):
         if graph_dt < dt:
             dt, launch = graph_dt, "hipgraph"
 
+    # The same stack driven through the C ABI alone (what a native host does: one oq_quantized_linear
+    # call per linear into buffers it owns, no module, no op dispatch, no allocation), to separate
+    # the library from the Python around it.  Reported beside `value`, not as `value`.
+    from orbitquant_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(device).cuda_stream
+    keep, calls = [], []
+    for l in mats:
+        x = x4096 if l.in_features == 4096 else x14336
+        nib = l.in_features // 2
+        bufs = (torch.empty((m, nib), dtype=torch.uint8, device=device), torch.empty(m, dtype=torch.float32, device=device),
+                torch.empty((m, l.out_features), dtype=torch.bfloat16, device=device))
+        keep.append(bufs)
+        calls.append((x.data_ptr(), 2, None, m, l.in_features, l._rotation_permutation.data_ptr(),
+                      l._rotation_signs.data_ptr(), l._activation_codebook_boundaries.data_ptr(),
+                      l._activation_codebook_centroids.data_ptr(), 4, l.rotation.block_size, l.activation_eps,
+                      l.rotation.normalization, l.packed_weight_indices.data_ptr(), l.weight_bits,
+                      l.row_norms.data_ptr(), l._weight_codebook_centroids.data_ptr(), None, 0, l.out_features,
+                      bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, stream))
+
+    def abi_step():
+        fn = lib.oq_quantized_linear
+        for c in calls:
+            if fn(*c) != 0:
+                raise RuntimeError(lib.oq_last_error().decode())
+    abi_step()
+    torch.cuda.synchronize()
+    assert torch.equal(keep[-1][2], mats[-1](x14336)), "C-ABI stack differs from the module stack"
+    abi_dt = time_steps(abi_step, args.steps, args.warmup)
+
     # kernel-only: every matmul launch of the stack, events on the launch stream
     per_stack = time_kernel(stack_matmuls, max(3, args.kernel_iters // 10))
     # W4 matrices alone (the 8 boundary layers' MLP up projections), cycled so the cache cannot hold them
@@ -485,6 +515,8 @@ def bench_c5(args, device):
                                         "packed_bytes_per_step": packed_bytes, "launch": launch,
                                         "eager_ms_per_step": eager_dt * 1e3,
                                         "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
+                                        "c_abi_ms_per_step": abi_dt * 1e3,
+                                        "c_abi_gbs": packed_bytes / abi_dt / 1e9,
                                         "preroll_s": PREROLL_SECONDS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("c5_gemv_w4_4096x14336"),
