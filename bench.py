@@ -37,9 +37,11 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
     ap.add_argument("--kernel-iters", type=int, default=50)
-    ap.add_argument("--unfused-activation", action="store_true",
-                    help="run the GELU between two linears as torch's separate kernel instead of handing it to "
-                         "the next layer's quantize kernel as a table (results are identical either way)")
+    ap.add_argument("--activation", default="output", choices=["output", "input", "separate"],
+                    help="where the GELU between two linears runs: as a table lookup in the epilogue of the "
+                         "matmul that produces its input (default), in the quantize kernel of the layer that "
+                         "consumes it, or as torch's separate kernel (identical results all three ways)")
+    ap.add_argument("--unfused-activation", action="store_true", help="same as --activation separate")
     return ap.parse_args()
 
 
@@ -94,7 +96,7 @@ def random_packed_weight(n, k, bits, gen, device):
     return packed.to(device)
 
 
-def build_layers(spec, device, gen, real_quantization: bool, fuse_activation: bool = True):
+def build_layers(spec, device, gen, real_quantization: bool, activation: str = "output"):
     from orbitquant_amd import OrbitLinear, OrbitQuantConfig
 
     layers = []
@@ -112,14 +114,19 @@ def build_layers(spec, device, gen, real_quantization: bool, fuse_activation: bo
         if layer.bias is not None:
             layer.bias.data = layer.bias.data.to(spec["dtype"])
         layers.append((layer, act))
-    if fuse_activation and spec["dtype"] in (torch.bfloat16, torch.float16):
-        for (_, act), (nxt, _) in zip(layers, layers[1:]):
-            if act == "gelu":   # the next layer's quantizer applies it (a table of torch's own GELU)
-                nxt.fuse_input_activation(torch.nn.functional.gelu, dtype=spec["dtype"])
+    if activation != "separate" and spec["dtype"] in (torch.bfloat16, torch.float16):
+        for (cur, act), (nxt, _) in zip(layers, layers[1:]):
+            if act == "gelu":   # a table of torch's own GELU, applied by one of the two layers around it
+                if activation == "output":
+                    cur.fuse_output_activation(torch.nn.functional.gelu, dtype=spec["dtype"])
+                else:
+                    nxt.fuse_input_activation(torch.nn.functional.gelu, dtype=spec["dtype"])
     return layers
 
 
 def activation_is_fused(layers, i) -> bool:
+    if layers[i][0]._output_activation_table is not None:
+        return True
     return i + 1 < len(layers) and layers[i + 1][0]._input_activation_table is not None
 
 
@@ -248,8 +255,9 @@ def _code_format(layer, x):
     return "u8" if (tokens > 16 and k % 64 == 0) or k % 128 == 0 else None
 
 
-def gemm_only_closure(layer, x):
-    """The matmul launch of `layer` alone, on pre-computed activation codes."""
+def gemm_only_closure(layer, x, with_output_map=True):
+    """The matmul launch of `layer` alone, on pre-computed activation codes (with the layer's
+    fused output activation, as it runs in the step, unless `with_output_map` is False)."""
     from orbitquant_amd import ops
 
     k = layer.in_features
@@ -267,7 +275,7 @@ def gemm_only_closure(layer, x):
                 codes, norms, layer._activation_codebook_centroids, layer.packed_weight_indices, layer.row_norms,
                 layer._weight_codebook_centroids, code_format=fmt, activation_bits=layer.activation_bits,
                 weight_bits=layer.weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
-                output_dtype=x.dtype)
+                output_dtype=x.dtype, output_map=layer._output_activation_table if with_output_map else None)
         return fn
     _, unit, norms = ops.rotate_quantize(
         x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
@@ -482,7 +490,7 @@ def bench_c5(args, device):
                       l._activation_codebook_centroids.data_ptr(), 4, l.rotation.block_size, l.activation_eps,
                       l.rotation.normalization, l.packed_weight_indices.data_ptr(), l.weight_bits,
                       l.row_norms.data_ptr(), l._weight_codebook_centroids.data_ptr(), None, 0, l.out_features,
-                      bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, stream))
+                      bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, None, stream))
 
     def abi_step():
         fn = lib.oq_quantized_linear
@@ -547,7 +555,7 @@ def main() -> int:
     spec = workload_spec(args.workload, args.m)
     gen = torch.Generator().manual_seed({"c1": 1, "c2": 2, "c3": 3, "c4": 4}[args.workload])
     real = args.workload in ("c1", "c2")        # larger workloads: synthetic indices (weight quantization is offline)
-    layers = build_layers(spec, device, gen, real, fuse_activation=not args.unfused_activation)
+    layers = build_layers(spec, device, gen, real, activation="separate" if args.unfused_activation else args.activation)
     x = make_input(spec, spec["layers"][0][0], gen).to(device)
     flops = sum(2.0 * spec["M"] * n * k for (k, n, *_rest) in spec["layers"])
 
@@ -572,6 +580,9 @@ def main() -> int:
         pieces[f"layer{i}"] = {
             "shape": [spec["M"], n, k], "gemm_us": tg * 1e6, "gemm_tflops": 2.0 * spec["M"] * n * k / tg / 1e12,
             "quantize_us": tq * 1e6, "quantize_gbs": q_bytes / tq / 1e9}
+        if layer._output_activation_table is not None:   # the same matmul without the activation in its epilogue
+            tp = time_kernel(gemm_only_closure(layer, h, with_output_map=False), args.kernel_iters)
+            pieces[f"layer{i}"]["gemm_us_without_activation"] = tp * 1e6
         h = apply_activation(layer(h), act, activation_is_fused(layers, i))
     dom = max(pieces.values(), key=lambda p: p["gemm_us"])
     achieved = dom["gemm_tflops"]
@@ -586,14 +597,21 @@ def main() -> int:
                    "flop_per_step": flops, "launch": launch, "eager_ms_per_step": eager_dt * 1e3,
                    "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
                    "preroll_s": PREROLL_SECONDS,
-                   "activation": ("gelu as a 65536-entry table of torch's own results inside the next layer's "
-                                  "quantize kernel" if any(activation_is_fused(layers, i) for i in range(len(layers)))
+                   "activation": ("gelu as a 65536-entry table of torch's own results, looked up in the producing "
+                                  "matmul's epilogue" if any(l._output_activation_table is not None for l, _ in layers)
+                                  else "gelu as a 65536-entry table of torch's own results, looked up in the next "
+                                  "layer's quantize kernel" if any(l._input_activation_table is not None for l, _ in layers)
                                   else "torch gelu kernel between the linears")},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded_traffic(f"{args.workload}_gemm"),
-                     "kernel": "packed_gemm_kernel", "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},
+                     "kernel": "packed_gemm_kernel" + (" with the GELU table in its epilogue"
+                                                       if "gemm_us_without_activation" in dom else ""),
+                     "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},
         "pieces": pieces,
     }
+    if "gemm_us_without_activation" in dom:
+        out["roofline"]["frac_without_activation"] = (2.0 * dom["shape"][0] * dom["shape"][1] * dom["shape"][2]
+                                                      / (dom["gemm_us_without_activation"] * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS)
     copy_calibration(device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, layers, x)

@@ -142,6 +142,21 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                      void *stream);
 
 /*
+ * oq_packed_linear followed by an elementwise function of the 16-bit outputs given as a
+ * table (output_map[bits of y] = bits of f(y), 65536 entries of the output dtype, 16-byte
+ * aligned, on the device): out = f(linear) bit for bit, f(...) applied before the store
+ * (tile kernels: in the epilogue; other kernels: by a small elementwise launch).  out_dtype
+ * must be OQ_F16 or OQ_BF16.  No counterpart in the reference, like oq_rotate_quantize_mapped:
+ * it is the activation that follows a linear, without its kernel.
+ */
+int oq_packed_linear_mapped(const void *codes, int code_format, const float *token_norms,
+                            const float *act_centroids, int a_bits,
+                            const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                            const float *w_centroids, const void *bias, int bias_dtype,
+                            int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
+                            const uint16_t *output_map, void *stream);
+
+/*
  * The whole quantized-linear forward in one call: oq_rotate_quantize (through
  * `input_map` when it is not NULL, see oq_rotate_quantize_mapped) followed by
  * oq_packed_linear, with the same results bit for bit.  It is the native form of the
@@ -154,6 +169,14 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
  * are not touched (they may be NULL).  Every other shape is the two launches, with the codes
  * ([M, K/2] bytes when a_bits <= 4 and K is even, else [M, K]) and norms (fp32 [M]) passing
  * through the caller's scratch buffers (16-byte aligned).
+ *
+ * `output_map` (NULL for none) is a table like `input_map`, of the OUTPUT dtype (16-bit
+ * only), applied to every output value before it is stored: out = f(linear(x)) bit for bit
+ * what f applied to the stored result of the plain call gives.  The tile kernels look the
+ * values up in their epilogue; the small-M and shape-agnostic kernels are followed by a tiny
+ * elementwise launch.  It is the cheaper place for the activation between two linears (a
+ * lookup per output value in a kernel that is waiting for its stores, instead of a lookup
+ * per input value in the quantizer, which has no such slack).
  */
 int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         int64_t M, int64_t K,
@@ -163,7 +186,7 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                         const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
                         void *codes_scratch, float *norms_scratch,
-                        void *out, int out_dtype, void *stream);
+                        void *out, int out_dtype, const uint16_t *output_map, void *stream);
 
 /*
  * Packed-weight matmul on float activations:

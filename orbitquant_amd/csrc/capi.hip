@@ -58,7 +58,8 @@ bool gemm_supported(int64_t K, int bits);
 int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                  int out_dtype, hipStream_t stream);
+                  int out_dtype, const uint16_t *out_map, hipStream_t stream);
+int apply_value_map(void *out, int64_t count, const uint16_t *table, hipStream_t stream);
 int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits);
 bool gemm_av_supported(int64_t K, int bits);
 int gemm_av_dispatch(bool f16, const void *a, const float *row_scale, const uint8_t *w, int bits,
@@ -125,28 +126,58 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
                                   input_map, as_stream(stream));
 }
 
-int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
-                     int a_bits, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
-                     const float *w_centroids, const void *bias, int bias_dtype, int64_t M, int64_t N,
-                     int64_t K, void *out, int out_dtype, void *stream) {
+// oq_packed_linear with an optional output map (applied by the tile kernels' epilogue, by a
+// small elementwise launch after the other kernels).
+static int packed_linear_impl(const void *codes, int code_format, const float *token_norms,
+                              const float *act_centroids, int a_bits, const uint8_t *packed_w, int w_bits,
+                              const uint16_t *row_norms, const float *w_centroids, const void *bias, int bias_dtype,
+                              int64_t M, int64_t N, int64_t K, void *out, int out_dtype, const uint16_t *out_map,
+                              void *stream) {
   if (int rc = check_matmul_common("packed_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
   if (M == 0) return OQ_OK;
   if (codes == nullptr || act_centroids == nullptr) return fail(OQ_ERR_INVALID, "packed_linear: null codes/centroids");
   if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "packed_linear: a_bits=%d", a_bits);
   if (code_format != OQ_CODES_U8 && code_format != OQ_CODES_NIBBLE) return fail(OQ_ERR_INVALID, "packed_linear: code_format=%d", code_format);
   if (code_format == OQ_CODES_NIBBLE && (a_bits > 4 || (K & 1))) return fail(OQ_ERR_INVALID, "packed_linear: nibble codes need a_bits <= 4 and even K");
+  if (out_map != nullptr) {
+    if (out_dtype == OQ_F32) return fail(OQ_ERR_INVALID, "packed_linear: an output map needs a 16-bit output dtype");
+    if (!aligned16(out_map)) return fail(OQ_ERR_INVALID, "packed_linear: the output map must be 16-byte aligned");
+  }
   const int a_levels = 1 << a_bits;
   hipStream_t s = as_stream(stream);
   const bool fast_ptrs = aligned16(codes) && aligned16(packed_w);
   const bool tiled_out = gemm_output_ok(N, out);  // the tiled kernels store 16-byte row segments
-  if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels))
-    return gemv_dispatch(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
-                         bias, bias_dtype, M, N, K, out, out_dtype, s);
-  if (fast_ptrs && tiled_out && gemm_supported(K, w_bits) && (code_format == OQ_CODES_NIBBLE || M > 16))
+  int rc;
+  if (fast_ptrs && gemv_supported(M, K, w_bits, code_format, a_levels)) {
+    rc = gemv_dispatch(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
+                       bias, bias_dtype, M, N, K, out, out_dtype, s);
+  } else if (fast_ptrs && tiled_out && gemm_supported(K, w_bits) && (code_format == OQ_CODES_NIBBLE || M > 16)) {
     return gemm_dispatch(code_format == OQ_CODES_NIBBLE ? 0 : 1, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
-                         bias, bias_dtype, M, N, K, out, out_dtype, s);
-  return generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
+                         bias, bias_dtype, M, N, K, out, out_dtype, out_map, s);
+  } else {
+    rc = generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
                               w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+  }
+  if (rc != OQ_OK || out_map == nullptr) return rc;
+  return apply_value_map(out, M * N, out_map, s);
+}
+
+int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
+                     int a_bits, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                     const float *w_centroids, const void *bias, int bias_dtype, int64_t M, int64_t N,
+                     int64_t K, void *out, int out_dtype, void *stream) {
+  return packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w, w_bits, row_norms,
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, nullptr, stream);
+}
+
+int oq_packed_linear_mapped(const void *codes, int code_format, const float *token_norms,
+                            const float *act_centroids, int a_bits, const uint8_t *packed_w, int w_bits,
+                            const uint16_t *row_norms, const float *w_centroids, const void *bias, int bias_dtype,
+                            int64_t M, int64_t N, int64_t K, void *out, int out_dtype, const uint16_t *output_map,
+                            void *stream) {
+  if (output_map == nullptr) return fail(OQ_ERR_INVALID, "packed_linear_mapped: output_map is null");
+  return packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w, w_bits, row_norms,
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
 }
 
 int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
@@ -154,19 +185,22 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
                         const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
                         const uint8_t *packed_w, int w_bits, const uint16_t *row_norms, const float *w_centroids,
                         const void *bias, int bias_dtype, int64_t N, void *codes_scratch, float *norms_scratch,
-                        void *out, int out_dtype, void *stream) {
+                        void *out, int out_dtype, const uint16_t *output_map, void *stream) {
   if (int rc = check_matmul_common("quantized_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
   if (M == 0) return OQ_OK;
   if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "quantized_linear: a_bits=%d", a_bits);
   if (act_centroids == nullptr) return fail(OQ_ERR_INVALID, "quantized_linear: null activation centroids");
   const int levels = 1 << a_bits;
   hipStream_t s = as_stream(stream);
+  if (output_map != nullptr && (out_dtype == OQ_F32 || !aligned16(output_map)))
+    return fail(OQ_ERR_INVALID, "quantized_linear: an output map needs a 16-bit output dtype and 16-byte alignment");
   if (aligned16(packed_w) && token_linear_supported(x_dtype, M, N, K, levels, w_bits, x, perm, signs)) {
     bool launched = false;
     const int rc = token_linear_dispatch(x, x_dtype, input_map, K, perm, signs, boundaries, act_centroids, levels, block,
                                          eps, inv_sqrt_block, packed_w, w_bits, row_norms, w_centroids, bias,
                                          bias_dtype, N, out, out_dtype, s, &launched);
-    if (rc != OQ_OK || launched) return rc;
+    if (rc != OQ_OK) return rc;
+    if (launched) return output_map == nullptr ? OQ_OK : apply_value_map(out, N, output_map, s);
   }
   if (codes_scratch == nullptr || norms_scratch == nullptr)
     return fail(OQ_ERR_INVALID, "quantized_linear: this shape takes two launches and needs the scratch buffers");
@@ -175,8 +209,8 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
                                         inv_sqrt_block, codes_scratch, fmt, nullptr, OQ_VALUES_NONE, norms_scratch,
                                         input_map, s))
     return rc;
-  return oq_packed_linear(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
-                          w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, stream);
+  return packed_linear_impl(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
 }
 
 int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,

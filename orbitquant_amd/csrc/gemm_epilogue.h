@@ -20,18 +20,34 @@
 // as the reads of step 2 have been issued.  The cost is instruction issue: about
 // 2.5 vector instructions per output value.
 //
+// An output map (the activation function that follows the linear, as a table) is applied
+// to the packed 16-bit words right before the store: a lookup in a 16 KB window of the
+// table kept in LDS behind the staging tiles, the full table in memory for the rare value
+// outside the window.
+//
 // Needs N % 8 == 0 and a 16-byte aligned `out` (the dispatcher sends other
 // shapes to the shape-agnostic kernels).
 #pragma once
 
+#include <type_traits>
+
 #include "packed_decode.h"
+#include "value_map.h"
 
 namespace oq {
 
 constexpr int kEpiFactorBytes = 3072;            // r_w[256] + bias[256] + token factor[256] as fp32
 constexpr int kEpiPitch = 64 * 4 + 16;           // one staged row: 64 fp32 + padding
 constexpr int kEpiWaveBytes = 32 * kEpiPitch;    // 8704
-constexpr int kEpiLdsBytes = kEpiFactorBytes + 4 * kEpiWaveBytes;
+constexpr int kEpiMapOffset = kEpiFactorBytes + 4 * kEpiWaveBytes;  // window of an output map (value_map.h)
+constexpr int kEpiLdsBytes = kEpiMapOffset + kWideBytes;
+
+// Optional elementwise function applied to the 16-bit outputs before they are stored, as a
+// table (value_map.h): table == nullptr means none; lo < 0 means no LDS window (fp16).
+struct OutMap {
+  const uint16_t *table;
+  int lo;
+};
 
 inline bool gemm_output_ok(int64_t N, const void *out) {
   return (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
@@ -82,8 +98,12 @@ template <int FM, int FN, int OUT_DT, bool GUARD>
 __device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN], int64_t m_tile, int64_t n_tile,
                                                     int wm, int wn, int tile_n, int tid, int64_t M, int64_t N,
                                                     const EpiFactors<FM> &pre, void *__restrict__ out,
-                                                    unsigned char *lds) {
+                                                    unsigned char *lds, const OutMap map) {
   const int lane = tid & 63, wave = tid >> 6, r = lane & 31, grp = lane >> 5;
+  const bool mapped = OUT_DT != OQ_F32 && map.table != nullptr;
+  uint16_t *hot_lds = reinterpret_cast<uint16_t *>(lds + kEpiMapOffset);
+  const uint16_t *hot = mapped && map.lo >= 0 ? hot_lds : nullptr;
+  if (hot != nullptr) fill_map_window<kWideLog2>(hot_lds, map.table, map.lo, tid, 256);  // published by the barrier below
 
   constexpr int ES = OUT_DT == OQ_F32 ? 4 : 2;
   float *rn_s = reinterpret_cast<float *>(lds);
@@ -142,25 +162,44 @@ __device__ __forceinline__ void gemm_epilogue_typed(const f32x16 (&acc)[FM][FN],
         sc[buf][t] = sc_s[wm + 32 * i + row];
       }
     };
-    auto finish = [&](int i, int buf) {
+    auto finish_groups = [&](int i, int buf, auto groups) {
+      constexpr int T = decltype(groups)::value;   // row groups of this tile: 32 / RPI
+      float y[kReads][8];
 #pragma unroll
-      for (int t = 0; t < 32 / RPI; ++t) {
+      for (int t = 0; t < T; ++t) {
         const float4 a0 = v0[buf][t], a1 = v1[buf][t];
         const float s = sc[buf][t];
-        const float y[8] = {(a0.x * s) * rn0.x + bv0.x, (a0.y * s) * rn0.y + bv0.y, (a0.z * s) * rn0.z + bv0.z,
-                            (a0.w * s) * rn0.w + bv0.w, (a1.x * s) * rn1.x + bv1.x, (a1.y * s) * rn1.y + bv1.y,
-                            (a1.z * s) * rn1.z + bv1.z, (a1.w * s) * rn1.w + bv1.w};
-        if (!GUARD || (col_ok && 32 * i + t * RPI < rows_left)) {
-          unsigned char *o = dst + (32 * i + t * RPI) * row_pitch;
-          if constexpr (OUT_DT == OQ_F32) {
-            reinterpret_cast<float4 *>(o)[0] = make_float4(y[0], y[1], y[2], y[3]);
-            reinterpret_cast<float4 *>(o)[1] = make_float4(y[4], y[5], y[6], y[7]);
-          } else {
-            *reinterpret_cast<uint4 *>(o) = make_uint4(pack_pair<OUT_DT>(y[0], y[1]), pack_pair<OUT_DT>(y[2], y[3]),
-                                                       pack_pair<OUT_DT>(y[4], y[5]), pack_pair<OUT_DT>(y[6], y[7]));
+        y[t][0] = (a0.x * s) * rn0.x + bv0.x; y[t][1] = (a0.y * s) * rn0.y + bv0.y;
+        y[t][2] = (a0.z * s) * rn0.z + bv0.z; y[t][3] = (a0.w * s) * rn0.w + bv0.w;
+        y[t][4] = (a1.x * s) * rn1.x + bv1.x; y[t][5] = (a1.y * s) * rn1.y + bv1.y;
+        y[t][6] = (a1.z * s) * rn1.z + bv1.z; y[t][7] = (a1.w * s) * rn1.w + bv1.w;
+      }
+      if constexpr (OUT_DT == OQ_F32) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          if (!GUARD || (col_ok && 32 * i + t * RPI < rows_left)) {
+            unsigned char *o = dst + (32 * i + t * RPI) * row_pitch;
+            reinterpret_cast<float4 *>(o)[0] = make_float4(y[t][0], y[t][1], y[t][2], y[t][3]);
+            reinterpret_cast<float4 *>(o)[1] = make_float4(y[t][4], y[t][5], y[t][6], y[t][7]);
           }
         }
+      } else {
+        uint4 words[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+          words[t] = make_uint4(pack_pair<OUT_DT>(y[t][0], y[t][1]), pack_pair<OUT_DT>(y[t][2], y[t][3]),
+                                pack_pair<OUT_DT>(y[t][4], y[t][5]), pack_pair<OUT_DT>(y[t][6], y[t][7]));
+        if (mapped) map_words8_many<OUT_DT, T, kWideLog2>(words, map.table, hot, map.lo);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          if (!GUARD || (col_ok && 32 * i + t * RPI < rows_left))
+            *reinterpret_cast<uint4 *>(dst + (32 * i + t * RPI) * row_pitch) = words[t];
+        }
       }
+    };
+    auto finish = [&](int i, int buf) {
+      if (JC == 2) finish_groups(i, buf, std::integral_constant<int, 4>{});
+      else finish_groups(i, buf, std::integral_constant<int, 2>{});
     };
     stage(0, 0);
 #pragma unroll
@@ -178,12 +217,13 @@ __device__ __forceinline__ void gemm_epilogue(const f32x16 (&acc)[FM][FN], int64
                                               int wn, int tile_n, int tid, int64_t M, int64_t N,
                                               const float *row_scale, const uint16_t *row_norms,
                                               const void *bias, int bias_dtype, const EpiFactors<FM> &pre,
-                                              void *out, int out_dtype, unsigned char *lds, int tile_m = 64 * FM) {
+                                              void *out, int out_dtype, unsigned char *lds, const OutMap map,
+                                              int tile_m = 64 * FM) {
   (void)row_scale; (void)row_norms; (void)bias; (void)bias_dtype;
   const bool interior = m_tile + tile_m <= M && n_tile + tile_n <= N;  // uniform over the workgroup
 #define OQ_EPILOGUE_CASE(DT)                                                                                   \
-  if (interior) gemm_epilogue_typed<FM, FN, DT, false>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds); \
-  else gemm_epilogue_typed<FM, FN, DT, true>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds)
+  if (interior) gemm_epilogue_typed<FM, FN, DT, false>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds, map); \
+  else gemm_epilogue_typed<FM, FN, DT, true>(acc, m_tile, n_tile, wm, wn, tile_n, tid, M, N, pre, out, lds, map)
   if (out_dtype == OQ_BF16) { OQ_EPILOGUE_CASE(OQ_BF16); }
   else if (out_dtype == OQ_F16) { OQ_EPILOGUE_CASE(OQ_F16); }
   else { OQ_EPILOGUE_CASE(OQ_F32); }

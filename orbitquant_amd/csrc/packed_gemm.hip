@@ -58,11 +58,12 @@ bool gemm_supported(int64_t K, int bits) {
 int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                  int out_dtype, hipStream_t stream) {
+                  int out_dtype, const uint16_t *out_map, hipStream_t stream) {
   GemmArgs g{};
   g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
+  g.out_map = OutMap{out_map, out_map != nullptr && out_dtype == OQ_BF16 ? kWideLoBf16 : -1};
   const int tile = gemm_choose_tile(M, N, K, bits);
   if (a_mode == A_NIBBLE) return launch_mode<A_NIBBLE>(g, bits, tile, stream);
   if (a_mode == A_U8) return gemm_launch_bytes(g, bits, tile, stream);

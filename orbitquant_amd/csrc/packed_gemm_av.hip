@@ -34,6 +34,7 @@ struct AvArgs {
   int64_t M, N, K;
   void *out;
   int out_dtype;
+  OutMap out_map;
   int tiles_m, tiles_n;
 };
 
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
 
   __syncthreads();  // tables and staging buffers are dead: LDS is reused by the epilogue
   gemm_epilogue<FM, FN>(acc, m0, n0, wm, wn, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
-                        g.out_dtype, reinterpret_cast<unsigned char *>(lds));
+                        g.out_dtype, reinterpret_cast<unsigned char *>(lds), g.out_map);
 }
 
 template <bool F16, int BITS, int FM, int FN>
@@ -235,6 +236,7 @@ int gemm_av_dispatch(bool f16, const void *a, const float *row_scale, const uint
   g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.w = w; g.row_norms = row_norms;
   g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype; g.M = M; g.N = N; g.K = K; g.out = out;
   g.out_dtype = out_dtype;
+  g.out_map = OutMap{nullptr, -1};
   return f16 ? launch_mode<true>(g, bits, tile, stream) : launch_mode<false>(g, bits, tile, stream);
 }
 

@@ -56,6 +56,7 @@ struct GemmArgs {
   int64_t M, N, K;
   void *out;
   int out_dtype;
+  OutMap out_map;            // optional elementwise function of the outputs (gemm_epilogue.h)
   int tiles_m, tiles_n;
 };
 
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   if constexpr (KSPLIT == 1) {
     gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, wn, TN, tid, g.M, g.N,
                           g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out, g.out_dtype,
-                          reinterpret_cast<unsigned char *>(lds));
+                          reinterpret_cast<unsigned char *>(lds), g.out_map);
   } else {
     // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
     // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
@@ -318,7 +319,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
       const f32x16 (&slice)[1][FN] = *reinterpret_cast<const f32x16 (*)[1][FN]>(&acc[W]);
       gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * W, 0, TN, tid, g.M,
                            g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
-                           reinterpret_cast<unsigned char *>(lds), TM);
+                           reinterpret_cast<unsigned char *>(lds), g.out_map, TM);
     };
     if (wave == 0) finish(std::integral_constant<int, 0>{});
     else if (wave == 1) finish(std::integral_constant<int, 1>{});

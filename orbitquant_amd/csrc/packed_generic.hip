@@ -118,4 +118,20 @@ int unpack_dispatch(const uint8_t *packed, int bits, int64_t count, uint8_t *out
   return check_launch("unpack_lowbit");
 }
 
+// out[i] = table[out[i]] for 16-bit outputs: the output map of the kernels that do not apply it
+// themselves (small-M and shape-agnostic paths, whose outputs are small).
+__global__ void apply_value_map_kernel(uint16_t *out, int64_t count, const uint16_t *table) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    out[i] = table[out[i]];
+}
+
+int apply_value_map(void *out, int64_t count, const uint16_t *table, hipStream_t stream) {
+  if (count <= 0) return OQ_OK;
+  const int64_t blocks = (count + 255) / 256;
+  hipLaunchKernelGGL(apply_value_map_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
+                     static_cast<uint16_t *>(out), count, table);
+  return check_launch("apply_value_map");
+}
+
 }  // namespace oq

@@ -108,7 +108,7 @@ int rotate_quantize_prepare(const void *x, int x_dtype, int64_t M, int64_t K, co
   RqArgs a;
   a.map = input_map;
   // bf16: |x| in [2^-10, 2^6) is served from LDS (exponent field 117 .. 132)
-  a.map_lo = (input_map != nullptr && x_dtype == OQ_BF16) ? (117 << 7) : -1;
+  a.map_lo = (input_map != nullptr && x_dtype == OQ_BF16) ? kHotLoBf16 : -1;
   a.map_lds_offset = 0;
   a.x = x; a.M = M; a.K = K; a.perm = perm; a.signs = signs; a.bounds = boundaries;
   a.cents = centroids; a.levels = levels;

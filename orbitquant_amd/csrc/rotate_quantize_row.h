@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "oq_common.h"
+#include "value_map.h"
 
 namespace oq {
 namespace rq {
@@ -60,51 +61,10 @@ struct RqArgs {
   int map_lds_offset;   // where the window starts in the dynamic LDS block (bytes, a multiple of 16)
 };
 
-constexpr int kHotHalf = 2048;                  // entries per sign: 16 binades of bf16
-constexpr int kHotBytes = 2 * kHotHalf * 2;     // 8 KB of LDS
-
-// The mapped value of eight 16-bit inputs.  bf16 inputs inside the window (|x| in 16 binades
-// chosen by the launcher, both signs) are served from the copy in LDS; a wavefront with any
-// input outside it also reads the full table in memory for those.  Other dtypes read the full
-// table for every input.
+// The mapped value of eight 16-bit inputs (value_map.h) for this kernel's arguments.
 template <int DT>
 __device__ __forceinline__ uint4 map_raw8(const uint4 raw, const RqArgs &a, const uint16_t *hot) {
-  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-  uint32_t out[4];
-  if (DT == OQ_BF16 && hot != nullptr) {
-    const uint32_t lo2 = static_cast<uint32_t>(a.map_lo) * 0x10001u;
-    uint32_t outside = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // per half: t = bits - lo (16-bit wrap); inside the window <=> (t & 0x7fff) < 2048; slot = (t & 0x7ff) + 2048 * sign
-      const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
-      outside |= t;
-      const uint32_t slot = (t & 0x07ff07ffu) | ((t >> 4) & 0x08000800u);
-      out[j] = static_cast<uint32_t>(hot[slot & 0xffffu]) | (static_cast<uint32_t>(hot[slot >> 16]) << 16);
-    }
-    if (__builtin_amdgcn_ballot_w64((outside & 0x78007800u) != 0) != 0) {
-      // all sixteen-bit loads are issued before any is used; inputs inside the window read entry 0 and drop it
-      uint32_t far[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
-        far[2 * j] = a.map[(t & 0x00007800u) ? (w[j] & 0xffffu) : 0u];
-        far[2 * j + 1] = a.map[(t & 0x78000000u) ? (w[j] >> 16) : 0u];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t t = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w[j]) - __builtin_bit_cast(u16x2, lo2));
-        if (t & 0x00007800u) out[j] = (out[j] & 0xffff0000u) | far[2 * j];
-        if (t & 0x78000000u) out[j] = (out[j] & 0x0000ffffu) | (far[2 * j + 1] << 16);
-      }
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      out[j] = static_cast<uint32_t>(a.map[w[j] & 0xffffu]) | (static_cast<uint32_t>(a.map[w[j] >> 16]) << 16);
-  }
-  return make_uint4(out[0], out[1], out[2], out[3]);
+  return map_words8<DT>(raw, a.map, hot, a.map_lo);
 }
 
 template <int DT, bool VEC>

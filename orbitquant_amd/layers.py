@@ -38,14 +38,14 @@ _LIB.define(
     "quantized_linear(Tensor x, Tensor permutation, Tensor signs, Tensor act_centroids, "
     "Tensor act_boundaries, Tensor packed_weight_indices, Tensor row_norms, Tensor weight_centroids, "
     "Tensor? bias, int block_size, float eps, float inv_sqrt_block, int activation_bits, "
-    "int weight_bits, int out_features, Tensor? input_map=None) -> Tensor"
+    "int weight_bits, int out_features, Tensor? input_map=None, Tensor? output_map=None) -> Tensor"
 )
 
 
 def quantized_linear_forward(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
-    input_map=None,
+    input_map=None, output_map=None,
 ):
     in_features = x.shape[-1]
     if bias is not None and bias.dtype != x.dtype:
@@ -58,21 +58,24 @@ def quantized_linear_forward(
             x, permutation, signs, act_boundaries, act_centroids, packed_weight_indices, row_norms,
             weight_centroids, block_size=block_size, eps=eps, inv_sqrt_block=inv_sqrt_block,
             activation_bits=activation_bits, weight_bits=weight_bits, out_features=out_features, bias=bias,
-            input_map=input_map)
+            input_map=input_map, output_map=output_map)
     _, unit, norms = ops.rotate_quantize(
         x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
         inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16",
         input_map=input_map)
-    return ops.matmul_packed_weight_values(
+    out = ops.matmul_packed_weight_values(
         unit, packed_weight_indices, row_norms, weight_centroids, bits=weight_bits,
         out_features=out_features, in_features=in_features, bias=bias,
         token_scale=norms.reshape(-1), output_dtype=x.dtype)
+    if output_map is not None:   # rare shapes only: plain gather through the table
+        out = output_map[out.view(torch.int16).to(torch.int32) & 0xFFFF]
+    return out
 
 
 def _quantized_linear_fake(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
-    input_map=None,
+    input_map=None, output_map=None,
 ):
     return x.new_empty((*x.shape[:-1], out_features))
 
@@ -124,6 +127,8 @@ class OrbitLinear(nn.Module):
         self.last_effective_runtime_mode: str | None = None
         self._input_activation = None  # (fn, dtype) once fuse_input_activation() was called
         self.register_buffer("_input_activation_table", None, persistent=False)
+        self._output_activation = None
+        self.register_buffer("_output_activation_table", None, persistent=False)
 
     def fuse_input_activation(self, fn, *, dtype: torch.dtype = torch.bfloat16) -> "OrbitLinear":
         """Make forward(x) return what forward(fn(x)) returns, bit for bit, without a separate
@@ -137,6 +142,20 @@ class OrbitLinear(nn.Module):
             return self
         self._input_activation = (fn, dtype)
         self._input_activation_table = ops.activation_table(fn, dtype, self.packed_weight_indices.device)
+        return self
+
+    def fuse_output_activation(self, fn, *, dtype: torch.dtype = torch.bfloat16) -> "OrbitLinear":
+        """Make forward(x) return fn(forward(x)), bit for bit, without a separate elementwise kernel:
+        fn (elementwise; the activation that follows this linear) is applied as a table lookup to every
+        output value right before it is stored.  This is the cheaper side to fuse an activation on
+        (the matmul's epilogue waits for its stores anyway); `fuse_input_activation` on the next layer is
+        for when this layer is not an OrbitLinear.  Inputs must have dtype `dtype`; `fn=None` undoes it."""
+        if fn is None:
+            self._output_activation = None
+            self._output_activation_table = None
+            return self
+        self._output_activation = (fn, dtype)
+        self._output_activation_table = ops.activation_table(fn, dtype, self.packed_weight_indices.device)
         return self
 
     def _constants(self) -> dict[str, torch.Tensor]:
@@ -178,6 +197,8 @@ class OrbitLinear(nn.Module):
         if self._input_activation is not None and device.type == "cuda":
             # a dtype cast must not touch the table's bits: fill it again
             self._input_activation_table = ops.activation_table(*self._input_activation, device)
+        if self._output_activation is not None and device.type == "cuda":
+            self._output_activation_table = ops.activation_table(*self._output_activation, device)
         return result
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -191,13 +212,16 @@ class OrbitLinear(nn.Module):
         table = self._input_activation_table
         if table is not None and table.dtype != x.dtype:
             raise ValueError(f"the fused input activation was built for {table.dtype}, got {x.dtype}")
+        out_table = self._output_activation_table
+        if out_table is not None and out_table.dtype != x.dtype:
+            raise ValueError(f"the fused output activation was built for {out_table.dtype}, got {x.dtype}")
         self.last_effective_runtime_mode = "hip_packed"
         return torch.ops.orbitquant_amd.quantized_linear(
             x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_centroids,
             self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
             self._weight_codebook_centroids, self.bias, self.rotation.block_size,
             self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
-            self.out_features, table)
+            self.out_features, table, out_table)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -161,6 +161,7 @@ def packed_linear(
     in_features: int,
     bias: torch.Tensor | None = None,
     output_dtype: torch.dtype = torch.bfloat16,
+    output_map: torch.Tensor | None = None,
 ) -> torch.Tensor:
     _require_gpu(codes, "codes")
     fmt = {"u8": OQ_CODES_U8, "nibble": OQ_CODES_NIBBLE}[code_format]
@@ -179,14 +180,22 @@ def packed_linear(
     norms = token_norms.reshape(-1)
     if norms.dtype != torch.float32 or norms.numel() != m:
         raise ValueError("token_norms must be float32 with one entry per token")
+    if output_map is not None:
+        if output_map.dtype != output_dtype or output_map.numel() != 65536 or output_map.device != codes.device \
+                or output_dtype == torch.float32:
+            raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on the codes' device")
+        output_map = output_map.contiguous()
     lib = _lib.load()
-    with _OnDevice(codes):
-        rc = lib.oq_packed_linear(
-            flat.data_ptr(), fmt, norms.contiguous().data_ptr(), activation_centroids.data_ptr(),
+    args = (flat.data_ptr(), fmt, norms.contiguous().data_ptr(), activation_centroids.data_ptr(),
             int(activation_bits), packed_weight_indices.data_ptr(), int(weight_bits),
             row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
             _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
-            out.data_ptr(), _DTYPES[output_dtype], _stream(codes))
+            out.data_ptr(), _DTYPES[output_dtype])
+    with _OnDevice(codes):
+        if output_map is None:
+            rc = lib.oq_packed_linear(*args, _stream(codes))
+        else:
+            rc = lib.oq_packed_linear_mapped(*args, output_map.data_ptr(), _stream(codes))
     _lib.check(rc, "oq_packed_linear")
     return out.reshape(*lead, out_features)
 
@@ -209,9 +218,12 @@ def quantized_linear(
     out_features: int,
     bias: torch.Tensor | None = None,
     input_map: torch.Tensor | None = None,
+    output_map: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """rotate_quantize followed by packed_linear in one native call (same results): a single
-    launch for one token of a 16-bit dtype (decode), two launches through scratch otherwise."""
+    launch for one token of a 16-bit dtype (decode), two launches through scratch otherwise.
+    input_map / output_map: tables (`activation_table`) of elementwise functions applied to the
+    input before it is quantized / to the output before it is stored."""
     _require_gpu(x, "x")
     dim = x.shape[-1]
     rows = x.contiguous().reshape(-1, dim)
@@ -231,6 +243,10 @@ def quantized_linear(
         if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device or x.dtype == torch.float32:
             raise ValueError("input_map must hold 65536 entries of x's 16-bit dtype on x's device")
         input_map = input_map.contiguous()
+    if output_map is not None:
+        if output_map.dtype != x.dtype or output_map.numel() != 65536 or output_map.device != x.device or x.dtype == torch.float32:
+            raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on x's device")
+        output_map = output_map.contiguous()
     if bias is not None:
         bias = bias.contiguous()
     nibble = activation_bits <= 4 and dim % 2 == 0
@@ -244,7 +260,7 @@ def quantized_linear(
             boundaries.data_ptr(), act_centroids.data_ptr(), int(activation_bits), int(block_size), float(eps),
             float(inv_sqrt_block), packed_weight.data_ptr(), int(weight_bits), row_norms.data_ptr(),
             weight_centroids.data_ptr(), _ptr(bias), _dt(bias) if bias is not None else 0, out_features,
-            codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _stream(x))
+            codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _ptr(output_map), _stream(x))
     _lib.check(rc, "oq_quantized_linear")
     return out.reshape(*x.shape[:-1], out_features)
 

@@ -122,7 +122,7 @@ def test_quantized_linear_argument_checks(dev):
             c["x"].data_ptr(), 2, None, m, 512, c["perm"].data_ptr(), c["signs"].data_ptr(), c["bounds"].data_ptr(),
             c["cents"].data_ptr(), a_bits, c["kw"]["block_size"], 1e-10, c["kw"]["inv_sqrt_block"],
             c["packed"].data_ptr(), 4, c["rn"].data_ptr(), c["wcents"].data_ptr(), None, 0, 256,
-            codes, norms, out.data_ptr(), 2, None)
+            codes, norms, out.data_ptr(), 2, None, None)
 
     assert call(2, None, None) == 1 and b"scratch" in lib.oq_last_error()   # two tokens need the scratch buffers
     assert call(1, None, None) == 0                                           # one token does not
