@@ -222,8 +222,14 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
   hipStream_t s = as_stream(stream);
   if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
+  {
+    // The float-activation kernel has its own (measured) preference: 256x256 tiles once there are
+    // at least half as many of them as CUs, 128x128 tiles below that; OQ_GEMM_TILE still overrides.
+    const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const int tile = getenv("OQ_GEMM_TILE") != nullptr ? gemm_choose_tile(M, N, K, bits) : (big_tiles >= 128 ? 2 : 0);
     return gemm_av_dispatch(x_dtype == OQ_F16, x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype,
-                            M, N, K, out, out_dtype, gemm_choose_tile(M, N, K, bits), s);
+                            M, N, K, out, out_dtype, tile, s);
+  }
   return generic_matmul_float(x, x_dtype, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N,
                               K, out, out_dtype, s);
 }
