@@ -23,6 +23,9 @@ int launch(const GemvArgs &g, hipStream_t stream) {
 
 template <bool BYTES, int BITS, int R>
 int launch_waves(const GemvArgs &g, int waves, hipStream_t stream) {
+  if constexpr (R == 1) {
+    if (waves == 16) return launch<BYTES, BITS, R, 16>(g, stream);
+  }
   if constexpr (!BYTES) {  // the other wavefront counts exist for experiments with OQ_GEMV_CFG only
     if (waves == 4) return launch<BYTES, BITS, R, 4>(g, stream);
     if (waves == 16) return launch<BYTES, BITS, R, 16>(g, stream);
@@ -33,7 +36,7 @@ int launch_waves(const GemvArgs &g, int waves, hipStream_t stream) {
 template <bool BYTES, int BITS>
 int launch_bits(const GemvArgs &g, hipStream_t stream) {
   // rows per workgroup (16*R) and K-split (wavefronts per workgroup); OQ_GEMV_CFG="R,WAVES" overrides
-  int r = g.N <= 16 * 512 ? 1 : 2, waves = 8;
+  int r = g.N <= 16 * 512 ? 1 : 2, waves = gemv_waves(g.N, g.K);
   if (const char *cfg = getenv("OQ_GEMV_CFG")) {
     int cr = 0, cw = 0;
     if (sscanf(cfg, "%d,%d", &cr, &cw) == 2 && (cr == 1 || cr == 2 || cr == 4) && (cw == 4 || cw == 8 || cw == 16)) {

@@ -52,6 +52,13 @@ struct GemvArgs {
 constexpr int kDepth = 1;  // K-steps of 128 fetched per batch of global loads (two batches in flight: decode of one overlaps the stream of the next)
 constexpr int kGemvTableBytes = kRowTableBytes;
 
+// Wavefronts per workgroup (= ways K is split).  When the whole launch is at most one workgroup
+// per CU (N <= 4096 with 16 rows each) eight wavefronts leave the CU's memory pipeline half
+// empty; sixteen measured 14-17 % faster there (4096x4096: 6.9 -> 5.9 us, 4096x14336:
+// 13.6 -> 11.3 us).  Rows shorter than 2048 do not have sixteen K-steps' worth of work.
+// The one-token kernel uses the same rule, so that both give the same sums.
+inline int gemv_waves(int64_t N, int64_t K) { return N <= 16 * 256 && K >= 2048 ? 16 : 8; }
+
 // BYTES: activation codes come one per byte (widths above 4 bits) instead of two per byte.
 // LATE: the activation codes and their row scales do not exist yet when the kernel starts;
 // `produce(issue_weights)`, called by every thread, writes them and calls `issue_weights()`
@@ -147,8 +154,9 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
   // ---- the packed stream first ------------------------------------------------------
   // Batches in flight: two for the plain stream (decode of one overlaps the loads of the next);
   // four when the activations come late, so that more of the weights are on their way while
-  // they are being produced (a wavefront's whole share for K up to 4096).
-  constexpr int NB = LATE ? 4 : 2;
+  // they are being produced (a wavefront's whole share for K up to 4096; with sixteen
+  // wavefronts two batches already are).
+  constexpr int NB = LATE && WAVES < 16 ? 4 : 2;  // sixteen wavefronts: half the K-steps each, and half the registers
   Batch b[NB];
   auto issue_weights = [&] {
 #pragma unroll

@@ -11,7 +11,6 @@ int token_linear_launch_w4(const rq::RqArgs &q, const gemv::GemvArgs &g, int x_d
 
 namespace {
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
-constexpr int kTokenThreads = 512;
 }  // namespace
 
 // One token, 16-bit input, nibble activation codes, a weight width the streaming kernel has a
@@ -42,7 +41,9 @@ int token_linear_dispatch(const void *x, int x_dtype, const uint16_t *input_map,
                                          OQ_VALUES_NONE, reinterpret_cast<float *>(16), input_map, &q, &vec);
   if (rc != OQ_OK) return rc;
   if (!vec) return OQ_OK;
-  const size_t rq_bytes = rq::lds_bytes(q, x_dtype, true, kTokenThreads / rq::kThreads);
+  // the quantizer runs on all wavefronts of the streaming workgroup: 2 or 4 groups of 256 threads
+  const int waves = N <= 16 * 256 ? gemv::gemv_waves(N, K) : 8;
+  const size_t rq_bytes = rq::lds_bytes(q, x_dtype, true, waves * 64 / rq::kThreads);
   const size_t dynamic = rq_bytes + K / 2 + 32;
   if (static_cast<size_t>(gemv::kGemvTableBytes) + dynamic > kLdsPerWorkgroup) return OQ_OK;  // the caller takes two launches
   gemv::GemvArgs g{};

@@ -14,12 +14,12 @@
 namespace oq {
 namespace {
 
-constexpr int kTokenWaves = 8;  // as the streaming kernel: 512 threads = two pass groups of the quantizer
-
 // Dynamic LDS: [0, codes_offset) is the quantizer's scratch, then K/2 bytes of nibble codes and
 // the norm (the streaming part's 64 KB table block is static).
-template <int DT, int LOG_G, int BITS, int R>
-__global__ __launch_bounds__(64 * kTokenWaves) void token_linear_kernel(rq::RqArgs q, gemv::GemvArgs g, int codes_offset) {
+// WAVES as the streaming kernel picks them (gemv_waves): 512 or 1024 threads = two or four pass
+// groups of the quantizer.
+template <int DT, int LOG_G, int BITS, int R, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void token_linear_kernel(rq::RqArgs q, gemv::GemvArgs g, int codes_offset) {
   extern __shared__ __align__(16) unsigned char smem[];
   uint8_t *codes = smem + codes_offset;
   float *norm = reinterpret_cast<float *>(codes + ((q.K / 2 + 15) & ~static_cast<int64_t>(15)));
@@ -28,25 +28,33 @@ __global__ __launch_bounds__(64 * kTokenWaves) void token_linear_kernel(rq::RqAr
   g.a = codes;
   g.row_scale = norm;
   const int tid = threadIdx.x;
-  gemv::packed_gemv_body<false, BITS, R, kTokenWaves, true>(g, [&](auto issue_weights) {
-    rq::rotate_quantize_row<DT, true, LOG_G, true>(q, smem, 0, tid, 64 * kTokenWaves, issue_weights);
+  gemv::packed_gemv_body<false, BITS, R, WAVES, true>(g, [&](auto issue_weights) {
+    rq::rotate_quantize_row<DT, true, LOG_G, true>(q, smem, 0, tid, 64 * WAVES, issue_weights);
   });
 }
 
-template <int DT, int LOG_G, int BITS, int R>
-int launch_token(const rq::RqArgs &q, const gemv::GemvArgs &g, size_t rq_bytes, hipStream_t stream) {
+template <int DT, int LOG_G, int BITS, int R, int WAVES>
+int launch_token_waves(const rq::RqArgs &q, const gemv::GemvArgs &g, size_t rq_bytes, hipStream_t stream) {
   const size_t scratch = rq_bytes;
   const size_t smem = scratch + static_cast<size_t>((q.K / 2 + 15) & ~static_cast<int64_t>(15)) + 16;
-  auto kern = token_linear_kernel<DT, LOG_G, BITS, R>;
+  auto kern = token_linear_kernel<DT, LOG_G, BITS, R, WAVES>;
   if (smem > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(smem)) != hipSuccess)
       return fail(OQ_ERR_LAUNCH, "token_linear: cannot reserve %zu bytes of LDS", smem);
   }
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * kTokenWaves), smem, stream, q, g,
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), smem, stream, q, g,
                      static_cast<int>(scratch));
   return check_launch("token_linear");
+}
+
+template <int DT, int LOG_G, int BITS, int R>
+int launch_token(const rq::RqArgs &q, const gemv::GemvArgs &g, size_t rq_bytes, hipStream_t stream) {
+  if constexpr (R == 1) {
+    if (gemv::gemv_waves(g.N, g.K) == 16) return launch_token_waves<DT, LOG_G, BITS, R, 16>(q, g, rq_bytes, stream);
+  }
+  return launch_token_waves<DT, LOG_G, BITS, R, 8>(q, g, rq_bytes, stream);
 }
 
 template <int DT, int BITS, int R>
