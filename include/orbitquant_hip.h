@@ -163,10 +163,12 @@ int oq_packed_linear_mapped(const void *codes, int code_format, const float *tok
  * reference layer's forward (src/orbitquant/layers.py:1079-1455: quantize_activations_*
  * then matmul_packed_*), which exists there only as Python glue between two ops.
  *
- * One token (M == 1) of a 16-bit dtype with a_bits <= 4 and w_bits 2, 3 or 4 is a SINGLE
- * launch: every workgroup of the streaming kernel quantizes the token itself while its first
- * weight loads are in flight, so decoding pays one launch per linear and the scratch buffers
- * are not touched (they may be NULL).  Every other shape is the two launches, with the codes
+ * One token (M == 1) of a 16-bit dtype with a_bits <= 4, w_bits 2, 3 or 4, K a multiple of
+ * 128 up to 8192, N up to 8192 and 16-byte aligned operands is a SINGLE launch: every workgroup
+ * of the streaming kernel quantizes the token itself while its weight loads are in flight, so
+ * decoding pays one launch per linear and the scratch buffers are not touched.  Callers that
+ * cannot tell in advance pass scratch always; NULL scratch is an error only when it is
+ * needed.  Every other shape is the two launches, with the codes
  * ([M, K/2] bytes when a_bits <= 4 and K is even, else [M, K]) and norms (fp32 [M]) passing
  * through the caller's scratch buffers (16-byte aligned).
  *
