@@ -28,6 +28,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "packed_decode.h"
 
 namespace oq {
@@ -100,7 +102,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
   auto fetch_a = [&](int s0, Batch &bt) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
-      const int s = min(s0 + d, s_end - 1);  // clamped: stays inside the row, result unused
+      const int s = max(min(s0 + d, s_end - 1), 0);  // clamped: stays inside the row, result unused
 #pragma unroll
       for (int v = 0; v < kAVec; ++v)
         bt.a[d][v] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * kAStep + 16 * v);
@@ -109,7 +111,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
   auto fetch_w = [&](int s0, Batch &bt) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
-      const int s = min(s0 + d, s_end - 1);
+      const int s = max(min(s0 + d, s_end - 1), 0);
 #pragma unroll
       for (int j = 0; j < R; ++j) load_w<BITS>(wp[j] + static_cast<int64_t>(s) * (16 * BITS), bt.w[d][j]);
     }
@@ -122,10 +124,10 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
   f32x4 acc[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  auto consume = [&](int s0, const Batch &bt) {
+  auto consume = [&](int s0, const Batch &bt, auto guarded) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
-      if (s0 + d < s_end) {
+      if (!decltype(guarded)::value || s0 + d < s_end) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           uint4 af;
@@ -160,13 +162,11 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
   Batch b[NB];
   auto issue_weights = [&] {
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      if (s_begin + i * kDepth < s_end) fetch_w(s_begin + i * kDepth, b[i]);
+    for (int i = 0; i < NB; ++i) fetch_w(s_begin + i * kDepth, b[i]);
   };
   if constexpr (!LATE) {
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      if (s_begin + i * kDepth < s_end) fetch(s_begin + i * kDepth, b[i]);
+    for (int i = 0; i < NB; ++i) fetch(s_begin + i * kDepth, b[i]);
   }
 
   // epilogue operands of the item this thread will finish (item = tid when tid < 64*R)
@@ -191,8 +191,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
     produce(issue_weights);
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
-      if (s_begin + i * kDepth < s_end) fetch_a(s_begin + i * kDepth, b[i]);
+    for (int i = 0; i < NB; ++i) fetch_a(s_begin + i * kDepth, b[i]);
     if (tid < 64 * R && ep_n < g.N) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -204,13 +203,23 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
     __syncthreads();
   }
 
-  for (int s = s_begin; s < s_end; s += NB * kDepth) {
+  // Every fetch is issued unconditionally (past the end of the wavefront's share it re-reads
+  // its last K-step, which the caches hold): the number of loads in flight is then the same on
+  // every path through the loop, and the wait before a batch is consumed is for that batch
+  // only.  With a fetch under a condition the compiler has to wait for every outstanding load
+  // at the top of the loop, and the stream stops while a batch is decoded.
+  int s = s_begin;
+  for (; s + NB * kDepth < s_end; s += NB * kDepth) {
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      if (s + i * kDepth < s_end) consume(s + i * kDepth, b[i]);
-      if (s + (NB + i) * kDepth < s_end) fetch(s + (NB + i) * kDepth, b[i]);
+      consume(s + i * kDepth, b[i], std::false_type{});
+      __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind its batch's decode
+      fetch(s + (NB + i) * kDepth, b[i]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
+#pragma unroll
+  for (int i = 0; i < NB; ++i) consume(s + i * kDepth, b[i], std::true_type{});
 
   // ---- cross-wave sum in LDS (the tables are dead), fixed order ------------------------
   __syncthreads();
