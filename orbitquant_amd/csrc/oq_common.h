@@ -53,6 +53,14 @@ __device__ __forceinline__ float load_dyn_f32(const void *p, int dt, int64_t i) 
   return load_as_f32<OQ_BF16>(p, i);
 }
 
+// Conversion of a value loaded as raw bits (a 16-bit pattern in the low half), for kernels that
+// request a value long before they use it.
+__device__ __forceinline__ float dyn_bits_to_f32(uint32_t b, int dt) {
+  if (dt == OQ_F32) return __builtin_bit_cast(float, b);
+  if (dt == OQ_F16) return f16_bits_to_f32(static_cast<uint16_t>(b));
+  return bf16_bits_to_f32(static_cast<uint16_t>(b));
+}
+
 __host__ __device__ inline int dtype_size(int dt) { return dt == OQ_F32 ? 4 : 2; }
 
 // index `v` of a little-endian bit stream, `bits` wide (1..8)

@@ -153,7 +153,28 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
     }
   };
 
-  // ---- the packed stream first ------------------------------------------------------
+  // Epilogue operands of the item this thread will finish (item = tid when tid < 64*R).  They
+  // are requested BEFORE the stream, by every thread, without a branch (clamped indices, a
+  // readable stand-in address for an absent operand) and stay untouched, as raw bits, until the
+  // epilogue.  A wavefront's loads return in order: a use of one of these values before the main
+  // loop - a conversion, or the register copy behind a value that is only loaded on one side of
+  // a branch - waits for every weight load issued before it, and did: the wavefronts that own
+  // an item used to start their table build only when their first weights had arrived.
+  const int ep_j = tid >> 6, ep_l = tid & 63;
+  const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
+  const int64_t ep_nc = min(ep_n, g.N - 1);
+  const bool has_bias = g.bias != nullptr, has_scale = !LATE && g.row_scale != nullptr;
+  const int bias_size = has_bias ? dtype_size(g.bias_dtype) : 2;
+  const uint8_t *bias_at = (has_bias ? static_cast<const uint8_t *>(g.bias) : reinterpret_cast<const uint8_t *>(g.row_norms)) + ep_nc * bias_size;
+  const uint32_t ep_rn_bits = g.row_norms[ep_nc];
+  const uint32_t ep_bias_lo = *reinterpret_cast<const uint16_t *>(bias_at);
+  const uint32_t ep_bias_hi = *reinterpret_cast<const uint16_t *>(bias_at + (bias_size - 2));
+  const float *scale_at = has_scale ? g.row_scale : g.w_cents;
+  float ep_sc_raw[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) ep_sc_raw[e] = scale_at[has_scale ? min(4 * (ep_l >> 4) + e, g.M - 1) : 0];
+
+  // ---- then the packed stream ------------------------------------------------------
   // Batches in flight: two for the plain stream (decode of one overlaps the loads of the next);
   // four when the activations come late, so that more of the weights are on their way while
   // they are being produced (a wavefront's whole share for K up to 4096; with sixteen
@@ -169,22 +190,6 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
     for (int i = 0; i < NB; ++i) fetch(s_begin + i * kDepth, b[i]);
   }
 
-  // epilogue operands of the item this thread will finish (item = tid when tid < 64*R)
-  const int ep_j = tid >> 6, ep_l = tid & 63;
-  const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
-  float ep_rn = 0.0f, ep_bv = 0.0f, ep_sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-  if (tid < 64 * R && ep_n < g.N) {
-    ep_rn = bf16_bits_to_f32(g.row_norms[ep_n]);
-    if (g.bias != nullptr) ep_bv = load_dyn_f32(g.bias, g.bias_dtype, ep_n);
-    if constexpr (!LATE) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int m = 4 * (ep_l >> 4) + e;
-        if (g.row_scale != nullptr && m < g.M) ep_sc[e] = g.row_scale[m];
-      }
-    }
-  }
-
   // ---- tables (built while the stream is in flight) ---------------------------------------
   build_row_tables<BITS, WAVES, BYTES>(lds, g.w_cents, g.act_cents, g.a_levels);
   if constexpr (LATE) {
@@ -192,13 +197,6 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < NB; ++i) fetch_a(s_begin + i * kDepth, b[i]);
-    if (tid < 64 * R && ep_n < g.N) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int m = 4 * (ep_l >> 4) + e;
-        if (g.row_scale != nullptr && m < g.M) ep_sc[e] = g.row_scale[m];
-      }
-    }
   } else {
     __syncthreads();
   }
@@ -236,11 +234,17 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce prod
       sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
     }
     const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+    const float ep_rn = bf16_bits_to_f32(static_cast<uint16_t>(ep_rn_bits));
+    const float ep_bv = has_bias ? dyn_bits_to_f32(bias_size == 4 ? (ep_bias_lo | (ep_bias_hi << 16)) : ep_bias_lo, g.bias_dtype) : 0.0f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int m = 4 * (ep_l >> 4) + e;
       if (m >= g.M) continue;
-      const float y = v[e] * ep_sc[e] * ep_rn + ep_bv;
+      float sc = has_scale ? ep_sc_raw[e] : 1.0f;
+      if constexpr (LATE) {  // produced by this launch: read where it is used
+        if (g.row_scale != nullptr) sc = g.row_scale[m];
+      }
+      const float y = v[e] * sc * ep_rn + ep_bv;
       const int64_t o = static_cast<int64_t>(m) * g.N + ep_n;
       if (g.out_dtype == OQ_BF16) static_cast<uint16_t *>(g.out)[o] = f32_to_bf16_bits(y);
       else if (g.out_dtype == OQ_F16) static_cast<uint16_t *>(g.out)[o] = f32_to_f16_bits(y);
