@@ -520,6 +520,9 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
           const uint32_t sw = e < 4 ? sg.x : sg.y;
           y[e] = __uint_as_float(__float_as_uint(y[e]) ^ ((sw << (24 - 8 * (e & 3))) & 0x80000000u));
         }
+      } else if constexpr (VEC) {  // K is a multiple of the chunk there: the whole chunk lies past the row
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) y[e] = 0.0f;
       } else {
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) {
