@@ -352,12 +352,25 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
   PermSigns ps_cur, ps_nxt;
   if constexpr (VEC) load_perm_signs(a, static_cast<int64_t>(pg) * kPass + t * kChunk, ps_cur);
 
-  // tables
+  // Tables: requested here, parked in LDS only after the row has been requested.  The loads are
+  // branch-free (clamped index, the boundaries as a readable stand-in for absent centroids) and
+  // their values are not touched before that, so nothing waits here: a wavefront's loads return
+  // in order, and a store of a loaded value at this point would put a full memory round trip
+  // in front of the row's own.
   const int nthreads = block_threads;  // 64 * (wavefronts that own a part of the row), or 256 * pass groups
-  for (int i = tid; i < 256; i += nthreads) {
-    bnd[i] = (i < a.levels - 1) ? a.bounds[i] : __builtin_inff();
-    cent[i] = (a.cents != nullptr && i < a.levels) ? a.cents[i] : 0.0f;
-  }
+  const float *cent_src = a.cents != nullptr ? a.cents : a.bounds;
+  const int cent_last = a.cents != nullptr ? a.levels - 1 : a.levels - 2;
+  // entry tid of the 256 (every entry a codebook of up to 64 levels has); the others, if any, at park time
+  const float table_b0 = a.bounds[min(tid, a.levels - 2)], table_c0 = cent_src[min(tid, cent_last)];
+  auto park_tables = [&] {
+    for (int i = tid; i < 256; i += nthreads) {
+      float bv = __builtin_inff(), cv = 0.0f;
+      if (i < a.levels - 1) bv = i == tid ? table_b0 : a.bounds[i];
+      if (a.cents != nullptr && i < a.levels) cv = i == tid ? table_c0 : a.cents[i];
+      bnd[i] = bv;
+      cent[i] = cv;
+    }
+  };
   if (tid == 0) cells_bad[0] = 0;
   if (windowed) {  // both signs of the window, 16 bytes per thread and step; the rows are mapped before the first barrier below
     for (int i = tid; i < kHotBytes / 16; i += nthreads) {
@@ -424,6 +437,7 @@ __device__ __forceinline__ void rotate_quantize_row(const RqArgs &a, unsigned ch
       square_sum(f, p);
     }
   }
+  park_tables();  // read after the barrier below
   if (groups_n > 1) {  // the lane's passes were summed by different threads: add them left to right
     __syncthreads();
     if (pg == 0) {
