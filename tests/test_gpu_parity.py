@@ -363,6 +363,23 @@ def test_packed_linear_small_m_stream_kernel(dev, m, n, k, wbits):
     assert torch.equal(got, again)      # fixed summation order: run-to-run identical
 
 
+@pytest.mark.parametrize("m", [1, 16])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize(("n", "k", "wbits"), [(64, 128, 4), (40, 256, 3), (100, 384, 2), (4104, 640, 4), (24, 1408, 4)])
+def test_packed_linear_small_m_short_rows(dev, m, n, k, wbits, with_bias, out_dtype):
+    """Rows of one to eleven K-steps: some wavefronts of a workgroup own no K-step at all, others an
+    odd number; bias absent, 16-bit and 32-bit (the kernel requests it long before it is used)."""
+    rng = np.random.default_rng(m + n + k + wbits)
+    layer = make_layer(rng, n, k, wbits, 4, with_bias=with_bias)
+    _, x32 = make_x(rng, m, k, torch.bfloat16, kind="plain")
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    want = oracle_linear(layer, codes, s, out_dtype)
+    got = run_packed_linear(dev, layer, codes, s, "nibble", out_dtype)
+    check_outputs(got.float().cpu().numpy(), want, s, layer["r"].float().numpy(), k, "small-M short rows")
+    assert torch.equal(got, run_packed_linear(dev, layer, codes, s, "nibble", out_dtype))
+
+
 @pytest.mark.parametrize("m", [1, 5, 16])
 @pytest.mark.parametrize(("n", "k", "wbits", "abits"), [(2048, 4096, 4, 6), (1000, 1024, 3, 8), (512, 1152, 6, 5), (4096, 4096, 2, 7)])
 def test_packed_linear_small_m_byte_codes(dev, m, n, k, wbits, abits):
