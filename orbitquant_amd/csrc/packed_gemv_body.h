@@ -16,7 +16,8 @@
 // Lookup tables: the 64 KB block of 256-byte rows the tiled GEMM uses (weight
 // entry e 32 times in bytes 0..127 of row e, activation entry e in bytes
 // 128..255; lane l reads copy l%32, a byte-indexed lookup is one v_perm_b32 plus
-// one ds_read_b32).  The packed stream is requested first thing; the tables are
+// one ds_read_b32).  The packed stream is requested first thing (right behind the few epilogue
+// operands, which are not touched before the epilogue); the tables are
 // built meanwhile from centroids fetched with SCALAR loads, which do not queue
 // behind the vector loads of the stream, and spread over the lanes so that every lane can pick the two values of its table entry with
 // wavefront shuffles.  After the main loop the same LDS holds the partial sums.
