@@ -128,7 +128,8 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
  * token_norms  fp32 [M]
  * act_centroids fp32 [2^a_bits]
  * packed_w     flat little-endian bit stream of idx[N,K], value v at bits [v*w_bits, v*w_bits+w_bits)
- *              (src/orbitquant/packing/bitpack.py:8-46); w_bits in {2,3,4,6,8}
+ *              (src/orbitquant/packing/bitpack.py:8-46); w_bits in [1, 8]: 2, 3, 4, 6 and 8 take the
+ *              tiled and streaming kernels, the other widths the shape-agnostic kernel
  * row_norms    bf16 [N] (raw uint16 bit patterns)
  * w_centroids  fp32 [2^w_bits]
  * bias         NULL or [N] of bias_dtype

@@ -4,6 +4,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "gemm_epilogue.h"
 
 namespace oq {
@@ -29,6 +33,30 @@ int check_launch(const char *what) {
   const hipError_t err = hipGetLastError();
   if (err != hipSuccess) return fail(OQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
   return OQ_OK;
+}
+
+bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
+  if (bytes <= 48 * 1024) return true;
+  static std::mutex lock;
+  static std::map<std::pair<const void *, int>, size_t> granted;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> guard(lock);
+  size_t &have = granted[std::make_pair(kernel, dev)];
+  if (bytes <= have) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) != hipSuccess) return false;
+  have = bytes;
+  return true;
+}
+
+const char *debug_env(int which) {
+  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG"};
+  static const char *values[ENV_COUNT];
+  static std::once_flag once;
+  std::call_once(once, [] {
+    for (int i = 0; i < ENV_COUNT; ++i) values[i] = getenv(names[i]);
+  });
+  return values[which];
 }
 
 // kernels (defined in the other translation units)
@@ -226,7 +254,7 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
     // The float-activation kernel has its own (measured) preference: 256x256 tiles once there are
     // at least half as many of them as CUs, 128x128 tiles below that; OQ_GEMM_TILE still overrides.
     const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    const int tile = getenv("OQ_GEMM_TILE") != nullptr ? gemm_choose_tile(M, N, K, bits) : (big_tiles >= 128 ? 2 : 0);
+    const int tile = debug_env(ENV_GEMM_TILE) != nullptr ? gemm_choose_tile(M, N, K, bits) : (big_tiles >= 128 ? 2 : 0);
     return gemm_av_dispatch(x_dtype == OQ_F16, x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype,
                             M, N, K, out, out_dtype, tile, s);
   }

@@ -12,6 +12,13 @@ namespace oq {
 void set_error(const char *fmt, ...);
 int fail(oq_status code, const char *fmt, ...);
 int check_launch(const char *what);
+// Dynamic LDS above 48 KB has to be granted per kernel: asks the runtime the first time a
+// (kernel, device) pair needs `bytes` or more than it was granted before, and answers from a
+// small table afterwards.  False if the runtime refuses.
+bool reserve_dynamic_lds(const void *kernel, size_t bytes);
+// Experiment switches (environment variables) are read once per process, at first use.
+const char *debug_env(int which);
+enum DebugEnv { ENV_GEMM_TILE = 0, ENV_NO_TOKEN_LINEAR, ENV_RQ_ONE_GROUP, ENV_GEMV_CFG, ENV_COUNT };
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

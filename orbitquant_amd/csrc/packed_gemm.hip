@@ -15,7 +15,7 @@ int gemm_launch_bytes(const GemmArgs &g, int bits, int tile, hipStream_t stream)
 // widths other than 4 pay for their longer index extraction, least on the largest tile.
 int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits) {
   const bool can_split = K % 256 == 0;  // a quarter of the K-steps per wavefront
-  const char *force = getenv("OQ_GEMM_TILE");
+  const char *force = debug_env(ENV_GEMM_TILE);
   if (force != nullptr && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
   if (force != nullptr && force[0] == '4' && can_split) return 4;
   struct Shape { int tm, tn; double fixed, step_short, step_busy, other_bits; };

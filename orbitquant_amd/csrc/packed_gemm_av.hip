@@ -145,8 +145,8 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
   }
   if (steps > 2) fetch_a(2);
   uint4 af0[FM], bf0[FN], af1[FM], bf1[FN];
+  __syncthreads();  // the lookup table (written by all threads above) and slab 0 are in LDS
   decode_b(0, bf0);
-  __syncthreads();
   read_a(0, 0, af0);
 
   // ---- main loop.  The barrier sits before the last of the four MFMA groups of a K-step, so
@@ -195,11 +195,8 @@ int launch_cfg(AvArgs g, hipStream_t stream) {
   size_t smem = WLut<BITS>::kDwords * sizeof(uint32_t) + 2 * static_cast<size_t>(TM) * kAPitch;
   if (smem < static_cast<size_t>(kEpiLdsBytes)) smem = kEpiLdsBytes;  // the epilogue reuses LDS
   auto kern = packed_gemm_av_kernel<F16, BITS, FM, FN>;
-  if (smem > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(smem)) != hipSuccess)
-      return fail(OQ_ERR_LAUNCH, "packed_gemm: cannot reserve %zu bytes of LDS", smem);
-  }
+  if (!reserve_dynamic_lds(reinterpret_cast<const void *>(kern), smem))
+    return fail(OQ_ERR_LAUNCH, "packed_gemm: cannot reserve %zu bytes of LDS", smem);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), smem, stream, g);
   return check_launch("packed_gemm_av");
 }

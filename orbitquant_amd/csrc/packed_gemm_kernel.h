@@ -288,43 +288,61 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
     // its own slice w.  Slot of destination s: [FN tiles][4 runs][64 lanes] of float4.
     float4 *slots = reinterpret_cast<float4 *>(lds);
-    auto finish = [&](auto wt) {
-      constexpr int W = decltype(wt)::value;
+    // The accumulator slices are registers, so which one a wavefront sends or keeps has to be a
+    // compile-time index: only the LDS traffic is selected per wavefront, every barrier (and
+    // the epilogue, which has one of its own) is reached by all four in the same place.
+    auto send = [&](auto wt, auto dt) __attribute__((always_inline)) {
+      constexpr int dst = (decltype(wt)::value + decltype(dt)::value) & 3;
 #pragma unroll
-      for (int d = 1; d < 4; ++d) {
-        const int dst = (W + d) & 3;
+      for (int j = 0; j < FN; ++j) {
+        const f32x16 t = acc[dst][j];  // whole-tile copies keep the accumulators in registers
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4)
-            slots[((dst * FN + j) * 4 + a4) * 64 + lane] = make_float4(acc[dst][j][4 * a4 + 0], acc[dst][j][4 * a4 + 1],
-                                                                       acc[dst][j][4 * a4 + 2], acc[dst][j][4 * a4 + 3]);
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int a4 = 0; a4 < 4; ++a4) {
-            const float4 v = slots[((W * FN + j) * 4 + a4) * 64 + lane];
-            acc[W][j][4 * a4 + 0] += v.x;
-            acc[W][j][4 * a4 + 1] += v.y;
-            acc[W][j][4 * a4 + 2] += v.z;
-            acc[W][j][4 * a4 + 3] += v.w;
-          }
-        __syncthreads();
+        for (int a4 = 0; a4 < 4; ++a4)
+          slots[((dst * FN + j) * 4 + a4) * 64 + lane] = make_float4(t[4 * a4 + 0], t[4 * a4 + 1], t[4 * a4 + 2], t[4 * a4 + 3]);
       }
-      EpiFactors<1> mine;
-      mine.rn = epi.rn;
-      mine.bv = epi.bv;
-      mine.sc[0] = epi.sc[W];
-      const f32x16 (&slice)[1][FN] = *reinterpret_cast<const f32x16 (*)[1][FN]>(&acc[W]);
-      gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * W, 0, TN, tid, g.M,
-                           g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
-                           reinterpret_cast<unsigned char *>(lds), g.out_map, TM);
     };
-    if (wave == 0) finish(std::integral_constant<int, 0>{});
-    else if (wave == 1) finish(std::integral_constant<int, 1>{});
-    else if (wave == 2) finish(std::integral_constant<int, 2>{});
-    else finish(std::integral_constant<int, 3>{});
+    // the last round's sum is the wavefront's own slice of the finished tile
+    f32x16 slice[1][FN];
+    EpiFactors<1> mine;
+    mine.rn = epi.rn;
+    mine.bv = epi.bv;
+    auto receive = [&](auto wt, auto dt) __attribute__((always_inline)) {
+      constexpr int W = decltype(wt)::value;
+      constexpr bool kLast = decltype(dt)::value == 3;
+      if constexpr (kLast) mine.sc[0] = epi.sc[W];
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        f32x16 t;
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+          const float4 v = slots[((W * FN + j) * 4 + a4) * 64 + lane];
+          t[4 * a4 + 0] = v.x;
+          t[4 * a4 + 1] = v.y;
+          t[4 * a4 + 2] = v.z;
+          t[4 * a4 + 3] = v.w;
+        }
+        if constexpr (kLast) slice[0][j] = acc[W][j] + t;
+        else acc[W][j] += t;
+      }
+    };
+#define OQ_KSPLIT_ROUND(D)                                                              \
+    if (wave == 0) send(std::integral_constant<int, 0>{}, std::integral_constant<int, D>{});      \
+    else if (wave == 1) send(std::integral_constant<int, 1>{}, std::integral_constant<int, D>{}); \
+    else if (wave == 2) send(std::integral_constant<int, 2>{}, std::integral_constant<int, D>{}); \
+    else send(std::integral_constant<int, 3>{}, std::integral_constant<int, D>{});                \
+    __syncthreads();                                                                    \
+    if (wave == 0) receive(std::integral_constant<int, 0>{}, std::integral_constant<int, D>{});      \
+    else if (wave == 1) receive(std::integral_constant<int, 1>{}, std::integral_constant<int, D>{}); \
+    else if (wave == 2) receive(std::integral_constant<int, 2>{}, std::integral_constant<int, D>{}); \
+    else receive(std::integral_constant<int, 3>{}, std::integral_constant<int, D>{});                \
+    __syncthreads();
+    OQ_KSPLIT_ROUND(1)
+    OQ_KSPLIT_ROUND(2)
+    OQ_KSPLIT_ROUND(3)
+#undef OQ_KSPLIT_ROUND
+    gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * wave, 0, TN, tid, g.M,
+                         g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
+                         reinterpret_cast<unsigned char *>(lds), g.out_map, TM);
   }
 }
 

@@ -37,7 +37,7 @@ template <bool BYTES, int BITS>
 int launch_bits(const GemvArgs &g, hipStream_t stream) {
   // rows per workgroup (16*R) and K-split (wavefronts per workgroup); OQ_GEMV_CFG="R,WAVES" overrides
   int r = g.N <= 16 * 512 ? 1 : 2, waves = gemv_waves(g.N, g.K);
-  if (const char *cfg = getenv("OQ_GEMV_CFG")) {
+  if (const char *cfg = debug_env(ENV_GEMV_CFG)) {
     int cr = 0, cw = 0;
     if (sscanf(cfg, "%d,%d", &cr, &cw) == 2 && (cr == 1 || cr == 2 || cr == 4) && (cw == 4 || cw == 8 || cw == 16)) {
       r = cr;

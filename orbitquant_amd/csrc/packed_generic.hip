@@ -28,7 +28,7 @@ struct GenericArgs {
   int out_dtype;
 };
 
-// grid = (N, ceil(M / kWaves)); block = 64 * kWaves; wave w handles row m = blockIdx.y*kWaves + w.
+// grid = (N, min(ceil(M / kWaves), 65535)); block = 64 * kWaves; wave w handles rows blockIdx.y*kWaves + w, + gridDim.y*kWaves, ...
 __global__ __launch_bounds__(64 * kWaves) void packed_generic_kernel(GenericArgs a) {
   __shared__ float wc[256];
   __shared__ float ac[256];
@@ -38,33 +38,35 @@ __global__ __launch_bounds__(64 * kWaves) void packed_generic_kernel(GenericArgs
   __syncthreads();
   const int lane = t & 63;
   const int64_t n = blockIdx.x;
-  const int64_t m = static_cast<int64_t>(blockIdx.y) * kWaves + (t >> 6);
-  if (m >= a.M) return;
   const int64_t nbytes = (a.N * a.K * a.bits + 7) / 8;
-  float acc = 0.0f;
-  for (int64_t k = lane; k < a.K; k += 64) {
-    const float w = wc[unpack_index(a.packed_w, n * a.K + k, a.bits, nbytes)];
-    float xv;
-    if (a.codes != nullptr) {
-      uint32_t code;
-      if (a.code_format == OQ_CODES_U8) code = a.codes[m * a.K + k];
-      else code = (a.codes[m * (a.K / 2) + (k >> 1)] >> ((k & 1) * 4)) & 0xfu;
-      xv = ac[code];
-    } else {
-      xv = load_dyn_f32(a.x, a.x_dtype, m * a.K + k);
+  // row groups beyond the grid's second dimension are walked by the same workgroups
+  for (int64_t m = static_cast<int64_t>(blockIdx.y) * kWaves + (t >> 6); m < a.M; m += static_cast<int64_t>(gridDim.y) * kWaves) {
+    float acc = 0.0f;
+    for (int64_t k = lane; k < a.K; k += 64) {
+      const float w = wc[unpack_index(a.packed_w, n * a.K + k, a.bits, nbytes)];
+      float xv;
+      if (a.codes != nullptr) {
+        uint32_t code;
+        if (a.code_format == OQ_CODES_U8) code = a.codes[m * a.K + k];
+        else code = (a.codes[m * (a.K / 2) + (k >> 1)] >> ((k & 1) * 4)) & 0xfu;
+        xv = ac[code];
+      } else {
+        xv = load_dyn_f32(a.x, a.x_dtype, m * a.K + k);
+      }
+      acc = fmaf(xv, w, acc);
     }
-    acc = fmaf(xv, w, acc);
-  }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (lane == 0) {
-    float y = acc * bf16_bits_to_f32(a.row_norms[n]);
-    if (a.token_scale != nullptr) y *= a.token_scale[m];
-    if (a.bias != nullptr) y += load_dyn_f32(a.bias, a.bias_dtype, n);
-    const int64_t o = m * a.N + n;
-    if (a.out_dtype == OQ_F32) store_from_f32<OQ_F32>(a.out, o, y);
-    else if (a.out_dtype == OQ_F16) store_from_f32<OQ_F16>(a.out, o, y);
-    else store_from_f32<OQ_BF16>(a.out, o, y);
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane == 0) {
+      // the same expression as the tiled and streaming kernels: (acc * token factor) * row norm + bias
+      float y = a.token_scale != nullptr ? acc * a.token_scale[m] : acc;
+      y = y * bf16_bits_to_f32(a.row_norms[n]);
+      if (a.bias != nullptr) y += load_dyn_f32(a.bias, a.bias_dtype, n);
+      const int64_t o = m * a.N + n;
+      if (a.out_dtype == OQ_F32) store_from_f32<OQ_F32>(a.out, o, y);
+      else if (a.out_dtype == OQ_F16) store_from_f32<OQ_F16>(a.out, o, y);
+      else store_from_f32<OQ_BF16>(a.out, o, y);
+    }
   }
 }
 
@@ -75,9 +77,9 @@ __global__ __launch_bounds__(256) void unpack_kernel(const uint8_t *packed, int 
 }
 
 int launch_generic(const GenericArgs &a, hipStream_t stream) {
-  if (a.N > 0x7fffffffLL || (a.M + kWaves - 1) / kWaves > 65535)
-    return fail(OQ_ERR_UNSUPPORTED, "generic packed kernel: M=%lld N=%lld exceed the grid", (long long)a.M, (long long)a.N);
-  dim3 grid(static_cast<unsigned>(a.N), static_cast<unsigned>((a.M + kWaves - 1) / kWaves));
+  if (a.N > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "generic packed kernel: N=%lld exceeds the grid", (long long)a.N);
+  const int64_t row_groups = (a.M + kWaves - 1) / kWaves;
+  dim3 grid(static_cast<unsigned>(a.N), static_cast<unsigned>(row_groups < 65535 ? row_groups : 65535));
   hipLaunchKernelGGL(packed_generic_kernel, grid, dim3(64 * kWaves), 0, stream, a);
   return check_launch("packed_generic");
 }

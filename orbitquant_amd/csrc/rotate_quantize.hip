@@ -19,7 +19,7 @@ int launch_for_block(const RqArgs &a, hipStream_t stream) {
   // a wavefront owns 512 consecutive elements of a pass: launch only the wavefronts a single-pass row needs
   const int waves = a.K >= 3 * kLaneSpan ? 4 : static_cast<int>((a.K + kLaneSpan - 1) / kLaneSpan);
   // few rows (decode): the chip is empty anyway, so run the passes of a long row side by side
-  const int pass_groups = (a.M <= 64 && a.passes >= 2 && getenv("OQ_RQ_ONE_GROUP") == nullptr) ? (a.passes >= 3 ? 4 : 2) : 1;
+  const int pass_groups = (a.M <= 64 && a.passes >= 2 && debug_env(ENV_RQ_ONE_GROUP) == nullptr) ? (a.passes >= 3 ? 4 : 2) : 1;
   dim3 grid(static_cast<unsigned>(a.M)), block(pass_groups > 1 ? kThreads * pass_groups : 64 * waves);
   RqArgs args = a;
   const size_t smem = lds_bytes(args, DT, VEC, pass_groups);
@@ -28,12 +28,8 @@ int launch_for_block(const RqArgs &a, hipStream_t stream) {
 #define OQ_RQ_LAUNCH(KERN)                                                                       \
   {                                                                                              \
     auto kern = KERN;                                                                            \
-    if (smem > 48 * 1024) {                                                                      \
-      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                              \
-                              hipFuncAttributeMaxDynamicSharedMemorySize,                        \
-                              static_cast<int>(smem)) != hipSuccess)                            \
-        return fail(OQ_ERR_LAUNCH, "rotate_quantize: cannot reserve %zu bytes of LDS", smem);    \
-    }                                                                                            \
+    if (!reserve_dynamic_lds(reinterpret_cast<const void *>(kern), smem))                        \
+      return fail(OQ_ERR_LAUNCH, "rotate_quantize: cannot reserve %zu bytes of LDS", smem);      \
     hipLaunchKernelGGL(kern, grid, block, smem, stream, args);                                   \
   }
 #define OQ_RQ_CASE(LG)                                                                           \

@@ -21,7 +21,7 @@ constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
 bool token_linear_supported(int x_dtype, int64_t M, int64_t N, int64_t K, int levels, int bits, const void *x,
                             const int32_t *perm, const int8_t *signs) {
   auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-  if (getenv("OQ_NO_TOKEN_LINEAR") != nullptr) return false;
+  if (debug_env(ENV_NO_TOKEN_LINEAR) != nullptr) return false;
   return M == 1 && (x_dtype == OQ_BF16 || x_dtype == OQ_F16) && levels <= 16 && K % 128 == 0 &&
          K <= 8192 && N <= 8192 && (bits == 2 || bits == 3 || bits == 4) &&
          aligned16(x) && aligned16(perm) && aligned16(signs);

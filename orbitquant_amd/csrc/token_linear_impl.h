@@ -38,11 +38,8 @@ int launch_token_waves(const rq::RqArgs &q, const gemv::GemvArgs &g, size_t rq_b
   const size_t scratch = rq_bytes;
   const size_t smem = scratch + static_cast<size_t>((q.K / 2 + 15) & ~static_cast<int64_t>(15)) + 16;
   auto kern = token_linear_kernel<DT, LOG_G, BITS, R, WAVES>;
-  if (smem > 48 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(smem)) != hipSuccess)
-      return fail(OQ_ERR_LAUNCH, "token_linear: cannot reserve %zu bytes of LDS", smem);
-  }
+  if (!reserve_dynamic_lds(reinterpret_cast<const void *>(kern), smem))
+    return fail(OQ_ERR_LAUNCH, "token_linear: cannot reserve %zu bytes of LDS", smem);
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), smem, stream, q, g,
                      static_cast<int>(scratch));

@@ -28,6 +28,26 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must live on an AMD GPU (torch device 'cuda'); got {t.device}")
 
 
+def _operand(t: torch.Tensor | None, name: str, like: torch.Tensor, *, dtype=None, numel: int | None = None,
+             min_numel: int | None = None) -> torch.Tensor | None:
+    """An auxiliary tensor whose raw pointer goes to the library: it must sit on `like`'s
+    device, have the expected dtype and element count, and is made contiguous."""
+    if t is None:
+        return None
+    if t.device != like.device:
+        raise ValueError(f"{name} is on {t.device}, the activations on {like.device}")
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if numel is not None and t.numel() != numel:
+        raise ValueError(f"{name} must hold {numel} elements, got {t.numel()}")
+    if min_numel is not None and t.numel() < min_numel:
+        raise ValueError(f"{name} must hold at least {min_numel} elements, got {t.numel()}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
 def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
@@ -84,10 +104,10 @@ def rotate_quantize(
     m = rows.shape[0]
     lead = x.shape[:-1]
     levels = boundaries.numel() + 1
-    if permutation.dtype != torch.int32 or signs.dtype != torch.int8:
-        raise ValueError("permutation must be int32 and signs int8")
-    if boundaries.dtype != torch.float32 or (centroids is not None and centroids.dtype != torch.float32):
-        raise ValueError("boundaries and centroids must be float32")
+    permutation = _operand(permutation, "permutation", x, dtype=torch.int32, numel=dim)
+    signs = _operand(signs, "signs", x, dtype=torch.int8, numel=dim)
+    boundaries = _operand(boundaries, "boundaries", x, dtype=torch.float32)
+    centroids = _operand(centroids, "centroids", x, dtype=torch.float32, numel=levels)
     codes = None
     fmt = OQ_CODES_U8
     if code_format == "u8":
@@ -171,22 +191,21 @@ def packed_linear(
     lead = codes.shape[:-1]
     flat = codes.contiguous().reshape(-1, width)
     m = flat.shape[0]
-    if row_norms.dtype != torch.bfloat16 or packed_weight_indices.dtype != torch.uint8:
-        raise ValueError("row_norms must be bfloat16 and packed_weight_indices uint8")
     expected = (out_features * in_features * weight_bits + 7) // 8
-    if packed_weight_indices.numel() < expected:
-        raise ValueError(f"packed_weight_indices holds {packed_weight_indices.numel()} bytes, needs {expected}")
+    packed_weight_indices = _operand(packed_weight_indices, "packed_weight_indices", codes, dtype=torch.uint8, min_numel=expected)
+    row_norms = _operand(row_norms, "row_norms", codes, dtype=torch.bfloat16, numel=out_features)
+    activation_centroids = _operand(activation_centroids, "activation_centroids", codes, dtype=torch.float32, numel=1 << activation_bits)
+    weight_centroids = _operand(weight_centroids, "weight_centroids", codes, dtype=torch.float32, numel=1 << weight_bits)
+    bias = _operand(bias, "bias", codes, dtype=_FLOATS, numel=out_features)
     out = torch.empty((m, out_features), dtype=output_dtype, device=codes.device)
-    norms = token_norms.reshape(-1)
-    if norms.dtype != torch.float32 or norms.numel() != m:
-        raise ValueError("token_norms must be float32 with one entry per token")
+    norms = _operand(token_norms.reshape(-1), "token_norms", codes, dtype=torch.float32, numel=m)
     if output_map is not None:
         if output_map.dtype != output_dtype or output_map.numel() != 65536 or output_map.device != codes.device \
                 or output_dtype == torch.float32:
             raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on the codes' device")
         output_map = output_map.contiguous()
     lib = _lib.load()
-    args = (flat.data_ptr(), fmt, norms.contiguous().data_ptr(), activation_centroids.data_ptr(),
+    args = (flat.data_ptr(), fmt, norms.data_ptr(), activation_centroids.data_ptr(),
             int(activation_bits), packed_weight_indices.data_ptr(), int(weight_bits),
             row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
             _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
@@ -228,17 +247,14 @@ def quantized_linear(
     dim = x.shape[-1]
     rows = x.contiguous().reshape(-1, dim)
     m = rows.shape[0]
-    if permutation.dtype != torch.int32 or signs.dtype != torch.int8:
-        raise ValueError("permutation must be int32 and signs int8")
-    if boundaries.dtype != torch.float32 or act_centroids.dtype != torch.float32 or weight_centroids.dtype != torch.float32:
-        raise ValueError("boundaries and centroids must be float32")
-    if boundaries.numel() + 1 != 1 << activation_bits:
-        raise ValueError("boundaries do not match activation_bits")
-    if row_norms.dtype != torch.bfloat16 or packed_weight.dtype != torch.uint8:
-        raise ValueError("row_norms must be bfloat16 and packed_weight uint8")
+    permutation = _operand(permutation, "permutation", x, dtype=torch.int32, numel=dim)
+    signs = _operand(signs, "signs", x, dtype=torch.int8, numel=dim)
+    boundaries = _operand(boundaries, "boundaries", x, dtype=torch.float32, numel=(1 << activation_bits) - 1)
+    act_centroids = _operand(act_centroids, "act_centroids", x, dtype=torch.float32, numel=1 << activation_bits)
+    weight_centroids = _operand(weight_centroids, "weight_centroids", x, dtype=torch.float32, numel=1 << weight_bits)
     expected = (out_features * dim * weight_bits + 7) // 8
-    if packed_weight.numel() != expected or row_norms.numel() != out_features:
-        raise ValueError(f"packed_weight must hold {expected} bytes and row_norms {out_features} values")
+    packed_weight = _operand(packed_weight, "packed_weight", x, dtype=torch.uint8, numel=expected)
+    row_norms = _operand(row_norms, "row_norms", x, dtype=torch.bfloat16, numel=out_features)
     if input_map is not None:
         if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device or x.dtype == torch.float32:
             raise ValueError("input_map must hold 65536 entries of x's 16-bit dtype on x's device")
@@ -247,8 +263,7 @@ def quantized_linear(
         if output_map.dtype != x.dtype or output_map.numel() != 65536 or output_map.device != x.device or x.dtype == torch.float32:
             raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on x's device")
         output_map = output_map.contiguous()
-    if bias is not None:
-        bias = bias.contiguous()
+    bias = _operand(bias, "bias", x, dtype=_FLOATS, numel=out_features)
     nibble = activation_bits <= 4 and dim % 2 == 0
     codes = torch.empty((m, dim // 2 if nibble else dim), dtype=torch.uint8, device=x.device)
     norms = torch.empty(m, dtype=torch.float32, device=x.device)
@@ -283,6 +298,12 @@ def matmul_packed_weight_values(
     flat = x.contiguous().reshape(-1, in_features)
     m = flat.shape[0]
     out_dtype = x.dtype if output_dtype is None else output_dtype
+    expected = (out_features * in_features * bits + 7) // 8
+    packed_weight_indices = _operand(packed_weight_indices, "packed_weight_indices", x, dtype=torch.uint8, min_numel=expected)
+    row_norms = _operand(row_norms, "row_norms", x, dtype=torch.bfloat16, numel=out_features)
+    weight_centroids = _operand(weight_centroids, "weight_centroids", x, dtype=torch.float32, numel=1 << bits)
+    bias = _operand(bias, "bias", x, dtype=_FLOATS, numel=out_features)
+    token_scale = _operand(token_scale, "token_scale", x, dtype=torch.float32, numel=m)
     out = torch.empty((m, out_features), dtype=out_dtype, device=x.device)
     lib = _lib.load()
     with _OnDevice(x):
@@ -297,6 +318,7 @@ def matmul_packed_weight_values(
 
 def unpack_lowbit(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
     _require_gpu(packed, "packed")
+    packed = _operand(packed, "packed", packed, dtype=torch.uint8, min_numel=(int(length) * int(bits) + 7) // 8)
     out = torch.empty(length, dtype=torch.uint8, device=packed.device)
     lib = _lib.load()
     with _OnDevice(packed):
