@@ -192,6 +192,31 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         void *out, int out_dtype, const uint16_t *output_map, void *stream);
 
 /*
+ * oq_quantized_linear for callers that cannot allocate device memory or bring a workspace:
+ * code running under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  Same arguments and same results as
+ * oq_quantized_linear, without the two scratch pointers: codes and norms pass through a buffer
+ * of OQ_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the library
+ * runs on holds its own copy until the process ends).  The call allocates and frees nothing.
+ * Shapes whose codes ([M, K/2] bytes for a_bits <= 4 and even K, else [M, K], rounded up to
+ * 256) plus norms (4 M bytes) do not fit are refused with OQ_ERR_UNSUPPORTED.  All calls on one
+ * GPU share the buffer: calls that may overlap there (different streams, or graphs replayed
+ * concurrently) race, and the buffer keeps the previous call's contents (every byte a call
+ * reads it has written itself first).  The buffer's address on a device is looked up the
+ * first time that device is current in oq_device_ok() or in this call; callers that capture
+ * graphs call oq_device_ok() once beforehand.
+ */
+#define OQ_STATIC_SCRATCH_BYTES (8u << 20)
+int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input_map,
+                               int64_t M, int64_t K,
+                               const int32_t *perm, const int8_t *signs,
+                               const float *boundaries, const float *act_centroids, int a_bits,
+                               int64_t block, float eps, float inv_sqrt_block,
+                               const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                               const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
+                               void *out, int out_dtype, const uint16_t *output_map, void *stream);
+
+/*
  * Packed-weight matmul on float activations:
  *
  *   out[m,n] = (sum_k x[m,k] * c_w[idx[n,k]]) * r_w[n] + bias[n]      (out in x's dtype)

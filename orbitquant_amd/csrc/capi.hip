@@ -99,6 +99,31 @@ int gemv_dispatch(const void *codes, int code_format, const float *row_scale, co
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream);
 
+// Scratch of oq_quantized_linear_static: the activation codes and token norms that pass from the
+// quantizer launch to the matmul launch.  One copy per GPU, at its own address there; host code
+// only ever uses the address hipGetSymbolAddress returns for the current device.
+constexpr size_t kStaticScratchBytes = OQ_STATIC_SCRATCH_BYTES;
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static int static_scratch_address(unsigned char **out) {
+  static std::mutex lock;
+  static unsigned char *address[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(OQ_ERR_LAUNCH, "no HIP device is current");
+  if (dev < 0 || dev >= kMaxDevices) return fail(OQ_ERR_UNSUPPORTED, "device index %d is beyond %d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> guard(lock);
+  if (address[dev] == nullptr) {
+    void *ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(OQ_ERR_LAUNCH, "cannot resolve the static scratch on device %d: %s", dev, hipGetErrorString(err));
+    address[dev] = static_cast<unsigned char *>(ptr);
+  }
+  *out = address[dev];
+  return OQ_OK;
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static bool valid_dtype(int dt) { return dt == OQ_F32 || dt == OQ_F16 || dt == OQ_BF16; }
 
@@ -131,7 +156,8 @@ int oq_device_ok(void) {
   if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return fail(OQ_ERR_LAUNCH, "cannot query device %d", dev);
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(OQ_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
-  return OQ_OK;
+  unsigned char *unused = nullptr;
+  return static_scratch_address(&unused);  // resolved here so that later calls (e.g. under graph capture) only look it up
 }
 
 int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
@@ -239,6 +265,29 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
     return rc;
   return packed_linear_impl(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
                             w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
+}
+
+int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
+                               const int32_t *perm, const int8_t *signs, const float *boundaries,
+                               const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
+                               const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                               const float *w_centroids, const void *bias, int bias_dtype, int64_t N, void *out,
+                               int out_dtype, const uint16_t *output_map, void *stream) {
+  if (M < 0 || K <= 0) return fail(OQ_ERR_INVALID, "quantized_linear_static: M=%lld K=%lld", (long long)M, (long long)K);
+  // layout of the scratch: codes (nibble or byte per value) rounded up to 256 bytes, then the norms
+  const bool nibble = a_bits <= 4 && (K & 1) == 0;
+  const uint64_t codes_bytes = static_cast<uint64_t>(M) * static_cast<uint64_t>(nibble ? K / 2 : K);
+  const uint64_t norms_at = (codes_bytes + 255u) & ~static_cast<uint64_t>(255);
+  if (static_cast<uint64_t>(K) > (1u << 20) || norms_at + 4u * static_cast<uint64_t>(M) > kStaticScratchBytes)
+    return fail(OQ_ERR_UNSUPPORTED,
+                "quantized_linear_static: %lld tokens of %lld values need %llu bytes of scratch, the static buffer holds %zu; "
+                "use oq_quantized_linear with caller-owned scratch",
+                (long long)M, (long long)K, (unsigned long long)(norms_at + 4u * static_cast<uint64_t>(M)), kStaticScratchBytes);
+  unsigned char *base = nullptr;
+  if (int rc = static_scratch_address(&base)) return rc;
+  return oq_quantized_linear(x, x_dtype, input_map, M, K, perm, signs, boundaries, act_centroids, a_bits, block, eps,
+                             inv_sqrt_block, packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, N, base,
+                             reinterpret_cast<float *>(base + norms_at), out, out_dtype, output_map, stream);
 }
 
 int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
