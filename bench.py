@@ -488,7 +488,7 @@ def bench_c5(args, device):
         calls.append((x.data_ptr(), 2, None, m, l.in_features, l._rotation_permutation.data_ptr(),
                       l._rotation_signs.data_ptr(), l._activation_codebook_boundaries.data_ptr(),
                       l._activation_codebook_centroids.data_ptr(), 4, l.rotation.block_size, l.activation_eps,
-                      l.rotation.normalization, l.packed_weight_indices.data_ptr(), l.weight_bits,
+                      l.rotation.normalization, l._rotation_plan.data_ptr(), l.packed_weight_indices.data_ptr(), l.weight_bits,
                       l.row_norms.data_ptr(), l._weight_codebook_centroids.data_ptr(), None, 0, l.out_features,
                       bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, None, stream))
 

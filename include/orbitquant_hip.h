@@ -79,6 +79,9 @@ const char *oq_version(void);
  * boundaries   fp32 [levels-1], ascending;  2 <= levels <= 256
  * centroids    fp32 [levels]; only read when values_mode != OQ_VALUES_NONE (else may be NULL)
  * block        power of two dividing K;  K <= 16384
+ * rotate_plan  NULL, or the plan oq_rotate_plan_build made from these perm, signs, boundaries,
+ *              levels, K, block and inv_sqrt_block: launches of more than 16 rows then take the
+ *              plan-based kernel (a third of the instructions, the same results bit for bit)
  * codes_out    NULL or [M, K] u8 / [M, K/2] u8 per code_format
  * values_out   NULL or per values_mode
  * norms_out    fp32 [M]: the raw norm s (no eps); may be NULL
@@ -86,10 +89,23 @@ const char *oq_version(void);
 int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K,
                        const int32_t *perm, const int8_t *signs,
                        const float *boundaries, const float *centroids, int levels,
-                       int64_t block, float eps, float inv_sqrt_block,
+                       int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan,
                        void *codes_out, int code_format,
                        void *values_out, int values_mode,
                        float *norms_out, void *stream);
+
+/*
+ * The rotate plan: everything the rotate+quantize kernel can know about a layer before it sees
+ * a token (permutation and signs merged into gather offsets, the boundaries folded with
+ * inv_sqrt_block, the bucketize table), built once per layer by one small launch and kept by
+ * the caller in device memory next to the layer's other constants: oq_rotate_plan_bytes(K)
+ * bytes, 16-byte aligned.  No counterpart in the reference, whose kernels re-derive all of it per
+ * row (packed_matmul.cu:581-657).  A plan is only valid for the arguments it was built from; a
+ * call that passes a plan built for another K, block or levels writes nothing.
+ */
+uint64_t oq_rotate_plan_bytes(int64_t K);
+int oq_rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *boundaries, int levels,
+                         int64_t K, int64_t block, float inv_sqrt_block, void *plan_out, void *stream);
 
 /*
  * The same, on f(x) instead of x, for an elementwise function f of a 16-bit
@@ -173,6 +189,8 @@ int oq_packed_linear_mapped(const void *codes, int code_format, const float *tok
  * ([M, K/2] bytes when a_bits <= 4 and K is even, else [M, K]) and norms (fp32 [M]) passing
  * through the caller's scratch buffers (16-byte aligned).
  *
+ * `rotate_plan` (NULL for none): see oq_rotate_quantize.
+ *
  * `output_map` (NULL for none) is a table like `input_map`, of the OUTPUT dtype (16-bit
  * only), applied to every output value before it is stored: out = f(linear(x)) bit for bit
  * what f applied to the stored result of the plain call gives.  The tile kernels look the
@@ -185,7 +203,7 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         int64_t M, int64_t K,
                         const int32_t *perm, const int8_t *signs,
                         const float *boundaries, const float *act_centroids, int a_bits,
-                        int64_t block, float eps, float inv_sqrt_block,
+                        int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan,
                         const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                         const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
                         void *codes_scratch, float *norms_scratch,
@@ -211,7 +229,7 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
                                int64_t M, int64_t K,
                                const int32_t *perm, const int8_t *signs,
                                const float *boundaries, const float *act_centroids, int a_bits,
-                               int64_t block, float eps, float inv_sqrt_block,
+                               int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan,
                                const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                                const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
                                void *out, int out_dtype, const uint16_t *output_map, void *stream);

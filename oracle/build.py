@@ -25,6 +25,11 @@ def build_oracle() -> Path:
         "-o", str(ORACLE_SO), str(HERE / "oq_oracle.c"), "-lm",
     ]
     subprocess.run(cmd, check=True)
+    checks = [
+        "gcc", "-O2", "-march=x86-64-v3", "-ffp-contract=off", "-fopenmp", "-shared", "-fPIC",
+        "-o", str(HERE / "liboq_kernel_checks.so"), str(HERE / "kernel_arith_check.c"), "-lm",
+    ]
+    subprocess.run(checks, check=True)
     return ORACLE_SO
 
 

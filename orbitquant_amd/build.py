@@ -29,6 +29,7 @@ COMMON = [
 SOURCES = {
     "capi.hip": [],
     "rotate_quantize.hip": ["-ffp-contract=off"],
+    "rotate_quantize_fast.hip": ["-ffp-contract=off"],
     "packed_generic.hip": [],
     "packed_gemm.hip": [],
     "packed_gemm_bytes.hip": [],

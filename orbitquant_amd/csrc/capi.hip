@@ -50,7 +50,7 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
 }
 
 const char *debug_env(int which) {
-  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG"};
+  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES"};
   static const char *values[ENV_COUNT];
   static std::once_flag once;
   std::call_once(once, [] {
@@ -64,7 +64,9 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              const int8_t *signs, const float *boundaries, const float *centroids,
                              int levels, int64_t block, float eps, float inv_sqrt_block,
                              void *codes_out, int code_format, void *values_out, int values_mode,
-                             float *norms_out, const uint16_t *input_map, hipStream_t stream);
+                             float *norms_out, const uint16_t *input_map, const void *plan, hipStream_t stream);
+int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *boundaries, int levels, int64_t K,
+                      int64_t block, float inv_sqrt_block, void *plan_out, hipStream_t stream);
 bool token_linear_supported(int x_dtype, int64_t M, int64_t N, int64_t K, int levels, int bits, const void *x,
                             const int32_t *perm, const int8_t *signs);
 int token_linear_dispatch(const void *x, int x_dtype, const uint16_t *input_map, int64_t K, const int32_t *perm,
@@ -162,11 +164,18 @@ int oq_device_ok(void) {
 
 int oq_rotate_quantize(const void *x, int x_dtype, int64_t M, int64_t K, const int32_t *perm,
                        const int8_t *signs, const float *boundaries, const float *centroids, int levels,
-                       int64_t block, float eps, float inv_sqrt_block, void *codes_out, int code_format,
-                       void *values_out, int values_mode, float *norms_out, void *stream) {
+                       int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan, void *codes_out,
+                       int code_format, void *values_out, int values_mode, float *norms_out, void *stream) {
   return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
                                   inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
-                                  nullptr, as_stream(stream));
+                                  nullptr, rotate_plan, as_stream(stream));
+}
+
+uint64_t oq_rotate_plan_bytes(int64_t K) { return K > 0 ? 3136u + 8u * static_cast<uint64_t>(K) : 0u; }
+
+int oq_rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *boundaries, int levels, int64_t K,
+                         int64_t block, float inv_sqrt_block, void *plan_out, void *stream) {
+  return rotate_plan_build(perm, signs, boundaries, levels, K, block, inv_sqrt_block, plan_out, as_stream(stream));
 }
 
 int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
@@ -177,7 +186,7 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
   if (input_map == nullptr) return fail(OQ_ERR_INVALID, "rotate_quantize_mapped: input_map is null");
   return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
                                   inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
-                                  input_map, as_stream(stream));
+                                  input_map, nullptr, as_stream(stream));
 }
 
 // oq_packed_linear with an optional output map (applied by the tile kernels' epilogue, by a
@@ -237,7 +246,7 @@ int oq_packed_linear_mapped(const void *codes, int code_format, const float *tok
 int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
                         const int32_t *perm, const int8_t *signs, const float *boundaries,
                         const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
-                        const uint8_t *packed_w, int w_bits, const uint16_t *row_norms, const float *w_centroids,
+                        const void *rotate_plan, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms, const float *w_centroids,
                         const void *bias, int bias_dtype, int64_t N, void *codes_scratch, float *norms_scratch,
                         void *out, int out_dtype, const uint16_t *output_map, void *stream) {
   if (int rc = check_matmul_common("quantized_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
@@ -261,7 +270,7 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
   const int fmt = (a_bits <= 4 && (K & 1) == 0) ? OQ_CODES_NIBBLE : OQ_CODES_U8;
   if (int rc = rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, nullptr, levels, block, eps,
                                         inv_sqrt_block, codes_scratch, fmt, nullptr, OQ_VALUES_NONE, norms_scratch,
-                                        input_map, s))
+                                        input_map, rotate_plan, s))
     return rc;
   return packed_linear_impl(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
                             w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
@@ -270,7 +279,7 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
 int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
                                const int32_t *perm, const int8_t *signs, const float *boundaries,
                                const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
-                               const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
+                               const void *rotate_plan, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                                const float *w_centroids, const void *bias, int bias_dtype, int64_t N, void *out,
                                int out_dtype, const uint16_t *output_map, void *stream) {
   if (M < 0 || K <= 0) return fail(OQ_ERR_INVALID, "quantized_linear_static: M=%lld K=%lld", (long long)M, (long long)K);
@@ -286,7 +295,7 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
   unsigned char *base = nullptr;
   if (int rc = static_scratch_address(&base)) return rc;
   return oq_quantized_linear(x, x_dtype, input_map, M, K, perm, signs, boundaries, act_centroids, a_bits, block, eps,
-                             inv_sqrt_block, packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, N, base,
+                             inv_sqrt_block, rotate_plan, packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, N, base,
                              reinterpret_cast<float *>(base + norms_at), out, out_dtype, output_map, stream);
 }
 

@@ -1,5 +1,6 @@
 // Fused RPBH rotate + per-token Lloyd-Max quantize for gfx950: the kernel (one workgroup per
 // token row), its launcher and the argument checks.  The arithmetic is in rotate_quantize_row.h.
+#include "rotate_plan.h"
 #include "rotate_quantize_row.h"
 
 namespace oq {
@@ -129,7 +130,20 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              const int8_t *signs, const float *boundaries, const float *centroids,
                              int levels, int64_t block, float eps, float inv_sqrt_block,
                              void *codes_out, int code_format, void *values_out, int values_mode,
-                             float *norms_out, const uint16_t *input_map, hipStream_t stream) {
+                             float *norms_out, const uint16_t *input_map, const void *plan, hipStream_t stream) {
+  // With a rotate plan, launches of more than a few rows take the plan-based kernel (same results);
+  // decode-sized launches and fused input maps stay with the kernel below, which is built for latency.
+  if (plan != nullptr && input_map == nullptr && M > 16) {
+    RqArgs checked;
+    bool vec_checked = false;
+    if (int rc = rotate_quantize_prepare(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
+                                         inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
+                                         input_map, &checked, &vec_checked))
+      return rc;
+    const int rc = rotate_quantize_fast(x, x_dtype, M, K, plan, levels, block, eps, centroids, codes_out, code_format,
+                                        values_out, values_mode, norms_out, stream);
+    if (rc >= 0) return rc;
+  }
   RqArgs a;
   bool vec = false;
   const int rc = rotate_quantize_prepare(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,

@@ -160,8 +160,8 @@ __device__ __forceinline__ int bucketize_cells(const uint2 *table, const CellMap
 }
 
 // Emit eight consecutive results (slots c0 .. c0+7 of `row`).
-template <int DT, bool VEC>
-__device__ __forceinline__ void emit8(const RqArgs &a, int64_t row, int64_t c0, const int (&code)[kChunk],
+template <int DT, bool VEC, typename Args>
+__device__ __forceinline__ void emit8(const Args &a, int64_t row, int64_t c0, const int (&code)[kChunk],
                                       const float *cent, float s) {
   const int64_t K = a.K;
   if (a.codes != nullptr) {

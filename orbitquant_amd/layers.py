@@ -38,14 +38,15 @@ _LIB.define(
     "quantized_linear(Tensor x, Tensor permutation, Tensor signs, Tensor act_centroids, "
     "Tensor act_boundaries, Tensor packed_weight_indices, Tensor row_norms, Tensor weight_centroids, "
     "Tensor? bias, int block_size, float eps, float inv_sqrt_block, int activation_bits, "
-    "int weight_bits, int out_features, Tensor? input_map=None, Tensor? output_map=None) -> Tensor"
+    "int weight_bits, int out_features, Tensor? input_map=None, Tensor? output_map=None, "
+    "Tensor? rotate_plan=None) -> Tensor"
 )
 
 
 def quantized_linear_forward(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
-    input_map=None, output_map=None,
+    input_map=None, output_map=None, rotate_plan=None,
 ):
     in_features = x.shape[-1]
     if bias is not None and bias.dtype != x.dtype:
@@ -58,11 +59,11 @@ def quantized_linear_forward(
             x, permutation, signs, act_boundaries, act_centroids, packed_weight_indices, row_norms,
             weight_centroids, block_size=block_size, eps=eps, inv_sqrt_block=inv_sqrt_block,
             activation_bits=activation_bits, weight_bits=weight_bits, out_features=out_features, bias=bias,
-            input_map=input_map, output_map=output_map)
+            input_map=input_map, output_map=output_map, plan=rotate_plan)
     _, unit, norms = ops.rotate_quantize(
         x, permutation, signs, act_boundaries, block_size=block_size, eps=eps,
         inv_sqrt_block=inv_sqrt_block, centroids=act_centroids, code_format=None, values="unit_bf16",
-        input_map=input_map)
+        input_map=input_map, plan=rotate_plan)
     out = ops.matmul_packed_weight_values(
         unit, packed_weight_indices, row_norms, weight_centroids, bits=weight_bits,
         out_features=out_features, in_features=in_features, bias=bias,
@@ -75,7 +76,7 @@ def quantized_linear_forward(
 def _quantized_linear_fake(
     x, permutation, signs, act_centroids, act_boundaries, packed_weight_indices, row_norms,
     weight_centroids, bias, block_size, eps, inv_sqrt_block, activation_bits, weight_bits, out_features,
-    input_map=None, output_map=None,
+    input_map=None, output_map=None, rotate_plan=None,
 ):
     return x.new_empty((*x.shape[:-1], out_features))
 
@@ -124,6 +125,8 @@ class OrbitLinear(nn.Module):
         device = packed_weight_indices.device
         for name, tensor in self._constants().items():
             self.register_buffer(name, tensor.to(device), persistent=False)
+        self.register_buffer("_rotation_plan", None, persistent=False)
+        self._build_rotation_plan()
         self.last_effective_runtime_mode: str | None = None
         self._input_activation = None  # (fn, dtype) once fuse_input_activation() was called
         self.register_buffer("_input_activation_table", None, persistent=False)
@@ -157,6 +160,16 @@ class OrbitLinear(nn.Module):
         self._output_activation = (fn, dtype)
         self._output_activation_table = ops.activation_table(fn, dtype, self.packed_weight_indices.device)
         return self
+
+    def _build_rotation_plan(self) -> None:
+        """What the quantize kernel can precompute from the layer's constants (`ops.rotate_plan`);
+        exists only while the module sits on a GPU."""
+        if self._rotation_permutation.device.type != "cuda":
+            self._rotation_plan = None
+            return
+        self._rotation_plan = ops.rotate_plan(
+            self._rotation_permutation, self._rotation_signs, self._activation_codebook_boundaries,
+            block_size=self.rotation.block_size, inv_sqrt_block=self.rotation.normalization)
 
     def _constants(self) -> dict[str, torch.Tensor]:
         return {
@@ -194,6 +207,7 @@ class OrbitLinear(nn.Module):
         device = self.packed_weight_indices.device
         for name, tensor in self._constants().items():
             setattr(self, name, tensor.to(device))
+        self._build_rotation_plan()
         if self._input_activation is not None and device.type == "cuda":
             # a dtype cast must not touch the table's bits: fill it again
             self._input_activation_table = ops.activation_table(*self._input_activation, device)
@@ -221,7 +235,7 @@ class OrbitLinear(nn.Module):
             self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
             self._weight_codebook_centroids, self.bias, self.rotation.block_size,
             self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
-            self.out_features, table, out_table)
+            self.out_features, table, out_table, self._rotation_plan)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -75,6 +75,33 @@ class _OnDevice:
         return False
 
 
+def rotate_plan(permutation: torch.Tensor, signs: torch.Tensor, boundaries: torch.Tensor, *, block_size: int,
+                inv_sqrt_block: float) -> torch.Tensor:
+    """The rotate plan of a layer (`oq_rotate_plan_build`): a uint8 blob on the constants' device
+    that `rotate_quantize(plan=...)` and `quantized_linear(plan=...)` take to run the plan-based
+    kernel.  Built by one small launch; valid for exactly these constants."""
+    _require_gpu(permutation, "permutation")
+    dim = permutation.numel()
+    permutation = _operand(permutation, "permutation", permutation, dtype=torch.int32)
+    signs = _operand(signs, "signs", permutation, dtype=torch.int8, numel=dim)
+    boundaries = _operand(boundaries, "boundaries", permutation, dtype=torch.float32)
+    lib = _lib.load()
+    plan = torch.empty(int(lib.oq_rotate_plan_bytes(dim)), dtype=torch.uint8, device=permutation.device)
+    with _OnDevice(permutation):
+        rc = lib.oq_rotate_plan_build(permutation.data_ptr(), signs.data_ptr(), boundaries.data_ptr(),
+                                      boundaries.numel() + 1, dim, int(block_size), float(inv_sqrt_block),
+                                      plan.data_ptr(), _stream(permutation))
+    _lib.check(rc, "oq_rotate_plan_build")
+    return plan
+
+
+def _plan_operand(plan: torch.Tensor | None, like: torch.Tensor, dim: int) -> torch.Tensor | None:
+    if plan is None:
+        return None
+    expected = int(_lib.load().oq_rotate_plan_bytes(dim))
+    return _operand(plan, "plan", like, dtype=torch.uint8, numel=expected)
+
+
 def rotate_quantize(
     x: torch.Tensor,
     permutation: torch.Tensor,
@@ -88,8 +115,12 @@ def rotate_quantize(
     code_format: str | None = "u8",
     values: str | None = None,
     input_map: torch.Tensor | None = None,
+    plan: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor | None, torch.Tensor | None, torch.Tensor]:
     """-> (codes or None, values or None, norms[...]).
+
+    plan: None, or `rotate_plan(...)` of the same permutation, signs, boundaries, block and
+    factor: more than 16 rows then take the plan-based kernel (same results, much faster).
 
     input_map: None, or the table of an elementwise function f (`activation_table`): the
     result is that of rotate_quantize(f(x)), bit for bit, without f(x) ever being stored.
@@ -136,15 +167,16 @@ def rotate_quantize(
         if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device:
             raise ValueError("input_map must hold 65536 entries of x's dtype on x's device")
         input_map = input_map.contiguous()
+    plan = _plan_operand(plan, x, dim)
     lib = _lib.load()
-    tail = (m, dim, permutation.data_ptr(), signs.data_ptr(), boundaries.data_ptr(), _ptr(centroids), levels,
-            int(block_size), float(eps), float(inv_sqrt_block), _ptr(codes), fmt, _ptr(out_values), mode,
-            norms.data_ptr(), _stream(x))
+    head = (m, dim, permutation.data_ptr(), signs.data_ptr(), boundaries.data_ptr(), _ptr(centroids), levels,
+            int(block_size), float(eps), float(inv_sqrt_block))
+    tail = (_ptr(codes), fmt, _ptr(out_values), mode, norms.data_ptr(), _stream(x))
     with _OnDevice(x):
         if input_map is None:
-            rc = lib.oq_rotate_quantize(rows.data_ptr(), _dt(rows), *tail)
+            rc = lib.oq_rotate_quantize(rows.data_ptr(), _dt(rows), *head, _ptr(plan), *tail)
         else:
-            rc = lib.oq_rotate_quantize_mapped(rows.data_ptr(), _dt(rows), input_map.data_ptr(), *tail)
+            rc = lib.oq_rotate_quantize_mapped(rows.data_ptr(), _dt(rows), input_map.data_ptr(), *head, *tail)
     _lib.check(rc, "oq_rotate_quantize")
     if codes is not None:
         codes = codes.reshape(*lead, codes.shape[-1])
@@ -238,6 +270,7 @@ def quantized_linear(
     bias: torch.Tensor | None = None,
     input_map: torch.Tensor | None = None,
     output_map: torch.Tensor | None = None,
+    plan: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """rotate_quantize followed by packed_linear in one native call (same results): a single
     launch for one token of a 16-bit dtype (decode), two launches through scratch otherwise.
@@ -264,6 +297,7 @@ def quantized_linear(
             raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on x's device")
         output_map = output_map.contiguous()
     bias = _operand(bias, "bias", x, dtype=_FLOATS, numel=out_features)
+    plan = _plan_operand(plan, x, dim)
     nibble = activation_bits <= 4 and dim % 2 == 0
     codes = torch.empty((m, dim // 2 if nibble else dim), dtype=torch.uint8, device=x.device)
     norms = torch.empty(m, dtype=torch.float32, device=x.device)
@@ -273,7 +307,7 @@ def quantized_linear(
         rc = lib.oq_quantized_linear(
             rows.data_ptr(), _dt(rows), _ptr(input_map), m, dim, permutation.data_ptr(), signs.data_ptr(),
             boundaries.data_ptr(), act_centroids.data_ptr(), int(activation_bits), int(block_size), float(eps),
-            float(inv_sqrt_block), packed_weight.data_ptr(), int(weight_bits), row_norms.data_ptr(),
+            float(inv_sqrt_block), _ptr(plan), packed_weight.data_ptr(), int(weight_bits), row_norms.data_ptr(),
             weight_centroids.data_ptr(), _ptr(bias), _dt(bias) if bias is not None else 0, out_features,
             codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _ptr(output_map), _stream(x))
     _lib.check(rc, "oq_quantized_linear")

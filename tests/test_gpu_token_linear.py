@@ -120,7 +120,7 @@ def test_quantized_linear_argument_checks(dev):
     def call(m, codes, norms, a_bits=4):
         return lib.oq_quantized_linear(
             c["x"].data_ptr(), 2, None, m, 512, c["perm"].data_ptr(), c["signs"].data_ptr(), c["bounds"].data_ptr(),
-            c["cents"].data_ptr(), a_bits, c["kw"]["block_size"], 1e-10, c["kw"]["inv_sqrt_block"],
+            c["cents"].data_ptr(), a_bits, c["kw"]["block_size"], 1e-10, c["kw"]["inv_sqrt_block"], None,
             c["packed"].data_ptr(), 4, c["rn"].data_ptr(), c["wcents"].data_ptr(), None, 0, 256,
             codes, norms, out.data_ptr(), 2, None, None)
 

@@ -62,7 +62,7 @@ def call(layer, x, *, static):
     stream = torch.cuda.current_stream(x.device).cuda_stream
     head = (x.data_ptr(), dt, None, m, k, layer["perm"].data_ptr(), layer["signs"].data_ptr(),
             layer["bounds"].data_ptr(), layer["cents"].data_ptr(), layer["abits"], layer["block"], 1e-10, layer["inv"],
-            layer["packed"].data_ptr(), layer["wbits"], layer["rn"].data_ptr(), layer["wcents"].data_ptr(),
+            layer["plan"].data_ptr() if layer.get("plan") is not None else None, layer["packed"].data_ptr(), layer["wbits"], layer["rn"].data_ptr(), layer["wcents"].data_ptr(),
             layer["bias"].data_ptr(), dt, n)
     if static:
         rc = lib.oq_quantized_linear_static(*head, out.data_ptr(), dt, None, stream)
