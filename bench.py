@@ -267,7 +267,7 @@ def gemm_only_closure(layer, x, with_output_map=True):
             x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
             block_size=layer.rotation.block_size, eps=layer.activation_eps,
             inv_sqrt_block=layer.rotation.normalization, code_format=fmt,
-            input_map=layer._input_activation_table)
+            input_map=layer._input_activation_table, plan=layer._rotation_plan)
         bias = layer.bias
 
         def fn():
@@ -303,7 +303,7 @@ def quantize_only_closure(layer, x):
             x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
             block_size=layer.rotation.block_size, eps=layer.activation_eps,
             inv_sqrt_block=layer.rotation.normalization, centroids=layer._activation_codebook_centroids,
-            code_format=fmt, values=vals, input_map=layer._input_activation_table)
+            code_format=fmt, values=vals, input_map=layer._input_activation_table, plan=layer._rotation_plan)
     return fn
 
 
@@ -407,6 +407,51 @@ def recorded_traffic(key: str):
 
 
 # ------------------------------------------------------------------------ c5
+
+def small_m_roofline(device, iters, m=1, copies=16):
+    """The small-M half of the metric on its roofline kernel: the streaming kernel on the W4
+    4096 -> 14336 matrix of the decode stack (29.4 MB of packed indices and row norms per launch),
+    timed alone with events on the launch stream, over `copies` distinct matrices launched in turn
+    (470 MB: more than the 256 MB of memory-side cache, so every launch streams from HBM)."""
+    from orbitquant_amd import ops
+    from orbitquant_amd.codebooks import get_codebook
+
+    k, n, bits = 4096, 14336, 4
+    gen = torch.Generator().manual_seed(55)
+    cb = get_codebook(k, bits)
+    cents = cb.centroids.to(device)
+    codes = torch.randint(0, 256, (m, k // 2), generator=gen, dtype=torch.uint8).to(device)
+    norms = torch.full((m,), 64.0, device=device)
+    row_norms = torch.full((n,), 1.28).to(torch.bfloat16).to(device)
+    mats = [torch.randint(0, 256, (n * k * bits // 8,), generator=gen, dtype=torch.uint8).to(device) for _ in range(copies)]
+
+    def fn():
+        for w in mats:
+            ops.packed_linear(codes, norms, cents, w, row_norms, cents, code_format="nibble", activation_bits=4,
+                              weight_bits=bits, out_features=n, in_features=k, output_dtype=torch.bfloat16)
+    per_launch = time_kernel(fn, max(3, iters // 5)) / copies
+    nbytes = mats[0].numel() + 2 * n
+    achieved = nbytes / per_launch / 1e9
+    return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": recorded_traffic("c5_gemv_w4_4096x14336"), "kernel": "packed_gemv_kernel<4> on 4096->14336 W4",
+            "M": m, "bytes_per_launch": nbytes, "avg_launch_us": per_launch * 1e6, "distinct_matrices": copies}
+
+
+def c3_gemm_lines(device, iters):
+    """The packed GEMMs of the Flux-style block (c3: W3A3, M = 4608), each timed alone: the other half
+    of "DiT-XL / Flux shapes" of the large-M target, reported beside the c2 headline."""
+    spec = workload_spec("c3", 0)
+    gen = torch.Generator().manual_seed(3)
+    layers = build_layers(spec, device, gen, False)
+    out = {}
+    for i, (layer, _act) in enumerate(layers):
+        k, n = layer.in_features, layer.out_features
+        x = make_input(spec, k, gen).to(device)
+        t = time_kernel(gemm_only_closure(layer, x), max(5, iters // 2))
+        tflops = 2.0 * spec["M"] * n * k / t / 1e12
+        out[f"{k}->{n}"] = {"gemm_us": t * 1e6, "gemm_tflops": tflops, "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
+    return out
+
 
 def build_c5(device, gen):
     """The 240 distinct matrices of the 40-layer decode stack: per layer q,k (4096x4096), v,o
@@ -526,11 +571,8 @@ def bench_c5(args, device):
                                         "c_abi_ms_per_step": abi_dt * 1e3,
                                         "c_abi_gbs": packed_bytes / abi_dt / 1e9,
                                         "preroll_s": PREROLL_SECONDS},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": recorded_traffic("c5_gemv_w4_4096x14336"),
-                     "kernel": "packed_gemv_kernel<4> on 4096->14336 W4", "bytes_per_launch": w4_bytes,
-                     "avg_launch_us": per_w4 * 1e6,
-                     "stack_matmuls_gbs": packed_bytes / per_stack / 1e9},
+        "roofline": dict(small_m_roofline(device, args.kernel_iters, m=m), stack_matmuls_gbs=packed_bytes / per_stack / 1e9,
+                         stack_w4_up_avg_launch_us=per_w4 * 1e6, stack_w4_up_gbs=achieved),
     }
     copy_calibration(device)
     print(json.dumps(out))
@@ -612,6 +654,10 @@ def main() -> int:
     if "gemm_us_without_activation" in dom:
         out["roofline"]["frac_without_activation"] = (2.0 * dom["shape"][0] * dom["shape"][1] * dom["shape"][2]
                                                       / (dom["gemm_us_without_activation"] * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS)
+    if args.workload == "c2":
+        # the two other figures the metric names, each on its own roofline kernel (`--workload c3|c5` for the full runs)
+        out["roofline_small_m"] = small_m_roofline(device, args.kernel_iters)
+        out["c3_gemms"] = c3_gemm_lines(device, args.kernel_iters)
     copy_calibration(device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, layers, x)

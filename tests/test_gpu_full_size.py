@@ -1,8 +1,10 @@
 """The configurations of the benchmark at their full sizes, through the layer's one-call entry
-point, checked on a sample of token rows: their activation codes must be the oracle's bit for
-bit and their outputs the oracle's within the path's bound.  The weights are random index
-bytes (what the matmul reads does not depend on how the indices were made); the oracle only
-ever sees the sampled rows, so each case takes seconds on the CPU."""
+point (which takes the plan-based quantizer for these sizes): EVERY activation code and token
+norm must be the oracle's bit for bit (the C oracle quantizes all rows, a few seconds per case
+on the host cores), and the outputs of a sample of token rows the oracle's within the path's
+bound.  The codebook tables are the reference generator's own (tests/golden/codebooks_v2.json).
+The weights are random index bytes (what the matmul reads does not depend on how the indices
+were made)."""
 
 from __future__ import annotations
 
@@ -13,6 +15,7 @@ import pytest
 import torch
 
 from oracle import oracle_c, oracle_np as o
+from parity_util import cosine, output_error, reference_tables
 
 pytestmark = pytest.mark.gpu
 
@@ -57,13 +60,13 @@ def activations(kind, m, k, gen):
 
 
 @pytest.mark.parametrize(("name", "m", "k", "n", "wbits", "abits", "kind"), FULL_SIZE)
-def test_full_size_layer_on_sampled_rows(dev, name, m, k, n, wbits, abits, kind):
+def test_full_size_layer(dev, name, m, k, n, wbits, abits, kind):
     from orbitquant_amd import ops
 
     gen = torch.Generator().manual_seed(1000 + m + k + n)
     perm, signs, block, inv = o.rpbh_constants(k, 0, "paper")
-    ca, ba = o.lloyd_max_tables(k, abits)
-    cw, _ = o.lloyd_max_tables(k, wbits)
+    ca, ba = reference_tables(k, abits)
+    cw, _ = reference_tables(k, wbits)
     packed = torch.randint(0, 256, ((n * k * wbits + 7) // 8,), generator=gen, dtype=torch.uint8)
     r = (0.02 * math.sqrt(k) * (1 + 0.05 * torch.randn(n, generator=gen))).to(torch.bfloat16)
     bias = (0.1 * torch.randn(n, generator=gen)).to(torch.bfloat16)
@@ -73,22 +76,27 @@ def test_full_size_layer_on_sampled_rows(dev, name, m, k, n, wbits, abits, kind)
     perm_d, signs_d = torch.from_numpy(perm.astype(np.int32)).to(dev), torch.from_numpy(signs).to(dev)
     ba_d, ca_d, cw_d = torch.from_numpy(ba).to(dev), torch.from_numpy(ca).to(dev), torch.from_numpy(cw).to(dev)
     kw = dict(block_size=block, eps=1e-10, inv_sqrt_block=float(inv))
+    plan = ops.rotate_plan(perm_d, signs_d, ba_d, block_size=block, inv_sqrt_block=float(inv))
     out = ops.quantized_linear(xd, perm_d, signs_d, ba_d, ca_d, packed.to(dev), r.to(dev), cw_d, activation_bits=abits,
-                               weight_bits=wbits, out_features=n, bias=bias.to(dev), **kw)
-    codes, _, norms = ops.rotate_quantize(xd, perm_d, signs_d, ba_d, code_format="u8", **kw)
+                               weight_bits=wbits, out_features=n, bias=bias.to(dev), plan=plan, **kw)
+    codes, _, norms = ops.rotate_quantize(xd, perm_d, signs_d, ba_d, code_format="u8", plan=plan, **kw)
+
+    # every code and norm of the launch
+    want_codes, want_s = oracle_c.rotate_quantize(x.float().numpy(), perm, signs, ba, block, 1e-10, inv)
+    got_codes = codes.cpu().numpy()
+    mismatches = int(np.count_nonzero(got_codes != want_codes))
+    assert mismatches == 0, f"{name}: {mismatches} of {got_codes.size} activation codes differ from the oracle"
+    assert np.array_equal(norms.cpu().numpy().view(np.int32), want_s.view(np.int32)), f"{name}: token norms differ from the oracle"
+    if m > 16:  # the plain kernel (what launches without a plan run) gives the same codes
+        codes_plain, _, norms_plain = ops.rotate_quantize(xd, perm_d, signs_d, ba_d, code_format="u8", **kw)
+        assert torch.equal(codes_plain, codes) and torch.equal(norms_plain, norms)
+    del got_codes
 
     rows = np.unique(np.concatenate([[0, m - 1], np.random.default_rng(m).integers(0, m, size=30)]))
-    sample = x[rows].float().numpy()
-    want_codes, want_s = oracle_c.rotate_quantize(sample, perm, signs, ba, block, 1e-10, inv)
-    assert np.array_equal(codes[rows].cpu().numpy(), want_codes), f"{name}: activation codes differ from the oracle"
-    assert np.array_equal(norms[rows].cpu().numpy(), want_s), f"{name}: token norms differ from the oracle"
-
-    want = oracle_c.linear_from_codes(want_codes, want_s, ca, packed.numpy(), wbits, r.float().numpy(), cw,
+    want = oracle_c.linear_from_codes(want_codes[rows], want_s[rows], ca, packed.numpy(), wbits, r.float().numpy(), cw,
                                       bias.float().numpy(), n)
-    got = out[rows].float().cpu().numpy().astype(np.float64)
-    bound = 2e-2 * want_s[:, None].astype(np.float64) * r.float().numpy()[None, :].astype(np.float64) / math.sqrt(k)
-    slack = np.abs(want) * 2.0 ** -8 + 1e-30   # the bf16 rounding of the output itself
-    worst = float((np.abs(got - want) / (bound + slack)).max())
-    assert worst <= 1.0, f"{name}: max error is {worst:.3f} of the bound"
-    cos = float((got * want).sum() / (np.linalg.norm(got) * np.linalg.norm(want) + 1e-300))
+    got = out[rows].float().cpu().numpy()
+    strict, rounded = output_error(got, want, want_s[rows], r.float().numpy(), k, True, True)
+    assert rounded <= 1.0, f"{name}: max error is {rounded:.3f} of the bound ({strict:.3f} without bf16's half-ulp)"
+    cos = cosine(got, want)
     assert cos >= 0.9999, f"{name}: cosine {cos}"

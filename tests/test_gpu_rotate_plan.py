@@ -28,7 +28,9 @@ def constants(dev, k, block, bits):
     from oracle import oracle_np
 
     perm, signs, h, inv = oracle_np.rpbh_constants(k, 0, block)
-    cents, bounds = oracle_np.lloyd_max_tables(k, bits)
+    from parity_util import reference_tables
+
+    cents, bounds = reference_tables(k, bits)
     t = dict(perm=torch.from_numpy(perm.astype(np.int32)).to(dev), signs=torch.from_numpy(signs.astype(np.int8)).to(dev),
              bounds=torch.from_numpy(bounds).to(dev), cents=torch.from_numpy(cents).to(dev))
     return perm, signs, h, inv, cents, bounds, t
