@@ -108,6 +108,31 @@ int oq_rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *
                          int64_t K, int64_t block, float inv_sqrt_block, void *plan_out, void *stream);
 
 /*
+ * The weight side of a layer on the GPU: what the packed matmuls read, made from a float weight
+ * matrix.  Replaces the reference's device-side weight quantization
+ * (src/orbitquant/layers.py:102-125,159-222; src/orbitquant/kernels/triton_cuda.py:926-1039,2740-2935).
+ * Per output row:
+ *
+ *   r      = ||fp32(w_row)||_2                     (the summation order of oq_rotate_quantize)
+ *   rot    = blockwise FWHT(fp32(w_row)[perm] * signs) * inv_sqrt_block
+ *   unit   = rot / max(r, eps)                     (IEEE division; note the order: rotate, scale, divide)
+ *   idx    = #{ j : boundaries[j] < unit }
+ *
+ * packed_out is the flat little-endian bit stream of idx[N, K], `bits` per index
+ * (ceil(N*K*bits/8) bytes; src/orbitquant/packing/bitpack.py:8-46), row_norms_out is bf16(r) [N].
+ * A zero row keeps r = 0, so it dequantizes to exact zeros.
+ *
+ * w            [N, K] of w_dtype, row-major, 16-byte aligned;  K a multiple of 8, K <= 16384
+ * rotate_plan  the plan oq_rotate_plan_build made from the layer's perm and signs with THESE
+ *              boundaries, levels, K, block and inv_sqrt_block (only its gather entries are used)
+ * boundaries   fp32 [levels-1] of the weight codebook;  2 <= levels <= 2^bits, 1 <= bits <= 8
+ * block        power of two dividing K, 8 <= block <= 4096
+ */
+int oq_quantize_weight(const void *w, int w_dtype, int64_t N, int64_t K, const void *rotate_plan,
+                       const float *boundaries, int levels, int64_t block, float eps, float inv_sqrt_block,
+                       int bits, uint8_t *packed_out, uint16_t *row_norms_out, void *stream);
+
+/*
  * The same, on f(x) instead of x, for an elementwise function f of a 16-bit
  * input given as a table: input_map[bits of x] = bits of f(x), 65536 entries of
  * the same dtype as x, 16-byte aligned, on the device.  The result is what

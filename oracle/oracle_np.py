@@ -250,14 +250,16 @@ def unpack_bits(packed, bits: int, count: int) -> np.ndarray:
 # weights and the linear itself
 # --------------------------------------------------------------------------
 
-def quantize_weight(weight, perm, signs, boundaries, block, eps, bits):
+def quantize_weight(weight, perm, signs, boundaries, block, eps, bits, norm_order="torch"):
     """layers.py:121-125,201-215 - (packed u8, row_norms bf16 as torch tensor, indices u8 [N,K]).
 
-    r = ||W_row|| on the unrotated fp32 row (torch.norm, as the reference);
-    rotW = rotate(W); unit = rotW / max(r, eps); idx = bucketize(unit).
+    r = ||W_row|| on the unrotated fp32 row; rotW = rotate(W); unit = rotW / max(r, eps);
+    idx = bucketize(unit).  norm_order "torch": torch.norm, as the reference's host path;
+    "sumsq_v1": the fixed order of `token_norms`, which is what the GPU kernel computes (the
+    reference's device path has an order of its own too, triton_cuda.py:150-152).
     """
     w = torch.as_tensor(np.asarray(weight, dtype=F32))
-    r = w.norm(dim=-1)
+    r = w.norm(dim=-1) if norm_order == "torch" else torch.from_numpy(token_norms(w.numpy()))
     rot = rotate(w.numpy(), perm, signs, block, F32(1.0 / math.sqrt(block)))
     unit = rot / np.maximum(r.numpy(), F32(eps))[:, None]
     idx = bucketize(unit, boundaries)

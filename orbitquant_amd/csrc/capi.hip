@@ -67,6 +67,9 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              float *norms_out, const uint16_t *input_map, const void *plan, hipStream_t stream);
 int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *boundaries, int levels, int64_t K,
                       int64_t block, float inv_sqrt_block, void *plan_out, hipStream_t stream);
+int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,
+                         int levels, int64_t block, float eps, float inv_sqrt_block, int bits, uint8_t *packed_out,
+                         uint16_t *row_norms_out, hipStream_t stream);
 bool token_linear_supported(int x_dtype, int64_t M, int64_t N, int64_t K, int levels, int bits, const void *x,
                             const int32_t *perm, const int8_t *signs);
 int token_linear_dispatch(const void *x, int x_dtype, const uint16_t *input_map, int64_t K, const int32_t *perm,
@@ -187,6 +190,14 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
   return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
                                   inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
                                   input_map, nullptr, as_stream(stream));
+}
+
+int oq_quantize_weight(const void *w, int w_dtype, int64_t N, int64_t K, const void *rotate_plan,
+                       const float *boundaries, int levels, int64_t block, float eps, float inv_sqrt_block, int bits,
+                       uint8_t *packed_out, uint16_t *row_norms_out, void *stream) {
+  const int rc = quantize_weight_fast(w, w_dtype, N, K, rotate_plan, boundaries, levels, block, eps, inv_sqrt_block, bits,
+                                      packed_out, row_norms_out, as_stream(stream));
+  return rc < 0 ? fail(OQ_ERR_UNSUPPORTED, "quantize_weight: no kernel for block %lld", (long long)block) : rc;
 }
 
 // oq_packed_linear with an optional output map (applied by the tile kernels' epilogue, by a

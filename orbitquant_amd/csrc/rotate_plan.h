@@ -64,4 +64,9 @@ int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const
                          float eps, const float *centroids, void *codes_out, int code_format, void *values_out,
                          int values_mode, float *norms_out, hipStream_t stream);
 
+// The weight side of a layer on the GPU (rotate_quantize_fast.hip): packed index stream + bf16 row norms.
+int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,
+                         int levels, int64_t block, float eps, float inv_sqrt_block, int bits, uint8_t *packed_out,
+                         uint16_t *row_norms_out, hipStream_t stream);
+
 }  // namespace oq

@@ -52,6 +52,12 @@ struct FastArgs {
   void *values;
   int values_mode;
   float *norms;
+  // EMIT_WEIGHT only
+  const float *raw_bounds;   // the codebook's boundaries as they are (the plan's are folded with 1/sqrt(block))
+  float inv_sqrt_block;
+  int pack_bits;
+  uint8_t *packed;           // flat bit stream of [M, K] indices
+  uint16_t *norms_bf16;      // [M]
 };
 
 // LDS: cells (2048) | thresholds (1024) | centroids (1024) | reduction slots (64) | staging
@@ -167,8 +173,12 @@ __device__ __forceinline__ void count_below(const uint2 (&ent)[kChunk], const fl
 }
 
 // What a launch writes: EMIT_NIBBLE / EMIT_U8 are the two hot forms (codes only), EMIT_ANY reads
-// the output arguments at run time (values modes, no codes, ...).
-enum EmitMode { EMIT_NIBBLE = 0, EMIT_U8 = 1, EMIT_ANY = 2 };
+// the output arguments at run time (values modes, no codes, ...).  EMIT_WEIGHT is the weight side
+// of the layer (src/orbitquant/layers.py:121-125,201-215 of the reference): the row is rotated
+// as it is, multiplied by 1/sqrt(block), THEN divided by max(norm, eps) with the IEEE division,
+// searched in the unfolded boundaries, and its indices are packed `pack_bits` wide into the flat
+// little-endian stream; the norm is stored as bf16.
+enum EmitMode { EMIT_NIBBLE = 0, EMIT_U8 = 1, EMIT_ANY = 2, EMIT_WEIGHT = 3 };
 
 // One row.  `smem`: fast_lds_bytes(K) bytes, 16-byte aligned.  All 64 * waves threads of the
 // workgroup make the call.
@@ -200,7 +210,8 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
   const int Ki = static_cast<int>(K);
   const int table_idx = min(tid, 255);
   const uint2 cell_v = reinterpret_cast<const uint2 *>(a.plan + plan::kCellsOffset)[table_idx];
-  const float thr_v = reinterpret_cast<const float *>(a.plan + plan::kThresholdsOffset)[table_idx];
+  const float thr_v = EMIT == EMIT_WEIGHT ? (table_idx < a.levels - 1 ? a.raw_bounds[table_idx] : __builtin_inff())
+                                          : reinterpret_cast<const float *>(a.plan + plan::kThresholdsOffset)[table_idx];
   const float cent_v = (EMIT == EMIT_ANY && a.cents != nullptr) ? a.cents[min(table_idx, a.levels - 1)] : 0.0f;
 
   // ---- phase A: stage the row (16-bit inputs as x and as -x), sum of squares -----------------
@@ -302,7 +313,8 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
 #pragma nounroll
   for (int idx = tid + nthreads; idx < 256; idx += nthreads) {  // workgroups of fewer than 256 threads only
     cells[idx] = reinterpret_cast<const uint2 *>(a.plan + plan::kCellsOffset)[idx];
-    thr[idx] = reinterpret_cast<const float *>(a.plan + plan::kThresholdsOffset)[idx];
+    thr[idx] = EMIT == EMIT_WEIGHT ? (idx < a.levels - 1 ? a.raw_bounds[idx] : __builtin_inff())
+                                   : reinterpret_cast<const float *>(a.plan + plan::kThresholdsOffset)[idx];
     cent[idx] = (EMIT == EMIT_ANY && a.cents != nullptr) ? a.cents[min(idx, a.levels - 1)] : 0.0f;
   }
   __syncthreads();
@@ -316,13 +328,17 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
 #pragma nounroll
   for (int w = 0; w < waves; ++w) row_plain = row_plain || red[4 + w] != 0.0f;
   if (tid == 0 && a.norms != nullptr) a.norms[row] = s_norm;
+  const float weight_denominator = s_norm < a.eps ? a.eps : s_norm;  // clamp_min(eps): a NaN norm stays NaN
+  if constexpr (EMIT == EMIT_WEIGHT) {
+    if (tid == 0) a.norms_bf16[row] = f32_to_bf16_bits(s_norm);
+  }
 
   // ---- phase B: units of max(H, 512) values, one wavefront each ---------------------------------
   // The two rare modes (IEEE division for this row, binary search instead of the cell table) pass
   // through an empty asm statement inside the loop on purpose: as loop invariants the compiler
   // clones the whole loop per combination.
   const uint32_t row_modes = __builtin_amdgcn_readfirstlane((row_plain ? 1u : 0u) | (hdr->cells != 0 ? 0u : 2u));
-  uint8_t *codes_row = a.codes + row * (EMIT == EMIT_NIBBLE ? K / 2 : K);  // uniform; EMIT_NIBBLE / EMIT_U8 only
+  uint8_t *codes_row = a.codes + row * (EMIT == EMIT_NIBBLE ? K / 2 : K);  // uniform; used by EMIT_NIBBLE / EMIT_U8 only
   const uint32_t neg1 = (lane & 1) ? 0x80000000u : 0u, neg2 = (lane & 2) ? 0x80000000u : 0u;
   // The gather entries of a step are requested one step ahead (past the last step: the row's
   // last chunk again, never used).
@@ -374,7 +390,10 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
           }
         }
       }
-      if (!plain) {
+      if constexpr (EMIT == EMIT_WEIGHT) {
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) y[j][e] = xv[e];
+      } else if (!plain) {
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) y[j][e] = divide_fast(xv[e], rc);
       } else {
@@ -409,7 +428,12 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
     for (int j = 0; j < G; ++j) {
       const int c0 = unit_base + j * kLaneSpan + lane_first;  // >= K: an idle lane of the row's last unit
       int code[kChunk];
-      if (!searched) {
+      if constexpr (EMIT == EMIT_WEIGHT) {
+        float unit[kChunk];
+#pragma unroll
+        for (int e = 0; e < kChunk; ++e) unit[e] = (y[j][e] * a.inv_sqrt_block) / weight_denominator;
+        rq::bucketize_many<kChunk>(thr, a.levels_pow2, unit, code);
+      } else if (!searched) {
         uint2 ent[kChunk];
 #pragma unroll
         for (int e = 0; e < kChunk; ++e) ent[e] = cells[plan::cell_of(y[j][e], cell_scale, cell_offset)];
@@ -428,6 +452,15 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
           w.x = ((((static_cast<uint32_t>(code[3]) << 8) | code[2]) << 8 | code[1]) << 8) | code[0];
           w.y = ((((static_cast<uint32_t>(code[7]) << 8) | code[6]) << 8 | code[5]) << 8) | code[4];
           *reinterpret_cast<uint2 *>(codes_row + static_cast<uint32_t>(c0)) = w;
+        } else if constexpr (EMIT == EMIT_WEIGHT) {
+          // eight indices = pack_bits whole bytes at a byte boundary of the stream (K is a multiple of 8)
+          uint64_t word = 0;
+#pragma unroll
+          for (int e = 0; e < kChunk; ++e) word |= static_cast<uint64_t>(code[e]) << (a.pack_bits * e);
+          uint8_t *dst = a.packed + (row * K + c0) / 8 * a.pack_bits;
+#pragma unroll
+          for (int b = 0; b < 8; ++b)
+            if (b < a.pack_bits) dst[b] = static_cast<uint8_t>(word >> (8 * b));
         } else {
           rq::emit8<DT, true>(a, row, c0, code, cent, s_norm);
         }

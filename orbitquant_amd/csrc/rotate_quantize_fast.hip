@@ -112,6 +112,7 @@ int launch_emit(const FastArgs &a, int waves, size_t smem, hipStream_t stream) {
 
 template <int DT, int LOG_H>
 int launch_one(const FastArgs &a, int waves, size_t smem, hipStream_t stream) {
+  if (a.packed != nullptr) return launch_emit<DT, LOG_H, EMIT_WEIGHT>(a, waves, smem, stream);
   if (a.codes != nullptr && a.values == nullptr) {
     if (a.code_format == OQ_CODES_NIBBLE) return launch_emit<DT, LOG_H, EMIT_NIBBLE>(a, waves, smem, stream);
     return launch_emit<DT, LOG_H, EMIT_U8>(a, waves, smem, stream);
@@ -154,6 +155,33 @@ int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *bou
   return check_launch("rotate_plan_build");
 }
 
+static int launch_fast(FastArgs &a, int x_dtype, hipStream_t stream);
+
+int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,
+                         int levels, int64_t block, float eps, float inv_sqrt_block, int bits, uint8_t *packed_out,
+                         uint16_t *row_norms_out, hipStream_t stream) {
+  auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  if (w == nullptr || plan == nullptr || boundaries == nullptr || packed_out == nullptr || row_norms_out == nullptr)
+    return fail(OQ_ERR_INVALID, "quantize_weight: null pointer");
+  if (w_dtype != OQ_F32 && w_dtype != OQ_F16 && w_dtype != OQ_BF16) return fail(OQ_ERR_INVALID, "quantize_weight: w_dtype=%d", w_dtype);
+  if (N < 0 || K <= 0) return fail(OQ_ERR_INVALID, "quantize_weight: N=%lld K=%lld", (long long)N, (long long)K);
+  if (bits < 1 || bits > 8 || levels < 2 || levels > (1 << bits))
+    return fail(OQ_ERR_INVALID, "quantize_weight: bits=%d levels=%d", bits, levels);
+  if (block <= 0 || (block & (block - 1)) != 0 || K % block != 0)
+    return fail(OQ_ERR_INVALID, "quantize_weight: block=%lld must be a power of two dividing K=%lld", (long long)block, (long long)K);
+  if (block < 8 || block > 4096 || K % 8 != 0 || K > 16384 || N > 0x7fffffffLL)
+    return fail(OQ_ERR_UNSUPPORTED, "quantize_weight: needs 8 <= block <= 4096, K a multiple of 8 up to 16384 (block=%lld K=%lld)",
+                (long long)block, (long long)K);
+  if (!aligned16(w) || !aligned16(plan)) return fail(OQ_ERR_INVALID, "quantize_weight: w and the plan must be 16-byte aligned");
+  if (N == 0) return OQ_OK;
+  FastArgs a{};
+  a.x = w; a.M = N; a.K = K; a.plan = static_cast<const unsigned char *>(plan);
+  a.levels = levels; a.block = static_cast<int>(block); a.eps = eps;
+  a.raw_bounds = boundaries; a.inv_sqrt_block = inv_sqrt_block; a.pack_bits = bits;
+  a.packed = packed_out; a.norms_bf16 = row_norms_out;
+  return launch_fast(a, w_dtype, stream);
+}
+
 int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const void *plan, int levels, int64_t block,
                          float eps, const float *centroids, void *codes_out, int code_format, void *values_out,
                          int values_mode, float *norms_out, hipStream_t stream) {
@@ -167,16 +195,24 @@ int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const
   a.x = x; a.M = M; a.K = K; a.plan = static_cast<const unsigned char *>(plan);
   a.cents = values_mode != OQ_VALUES_NONE ? centroids : nullptr;
   a.levels = levels;
-  a.levels_pow2 = 2;
-  while (a.levels_pow2 < levels) a.levels_pow2 <<= 1;
   a.block = static_cast<int>(block);
-  a.passes = static_cast<int>((K + kPass - 1) / kPass);
-  const int64_t unit = block > kLaneSpan ? block : kLaneSpan;
-  a.units = static_cast<int>((K + unit - 1) / unit);
   a.eps = eps;
   a.codes = static_cast<uint8_t *>(codes_out); a.code_format = code_format;
   a.values = values_mode == OQ_VALUES_NONE ? nullptr : values_out; a.values_mode = values_mode;
   a.norms = norms_out;
+  return launch_fast(a, x_dtype, stream);
+}
+
+// Derived launch parameters and the launch itself; -1 when no kernel is instantiated for the block size.
+static int launch_fast(FastArgs &a, int x_dtype, hipStream_t stream) {
+  const int64_t K = a.K, block = a.block;
+  int log_h = 0;
+  while ((int64_t{1} << log_h) < block) ++log_h;
+  a.levels_pow2 = 2;
+  while (a.levels_pow2 < a.levels) a.levels_pow2 <<= 1;
+  a.passes = static_cast<int>((K + kPass - 1) / kPass);
+  const int64_t unit = block > kLaneSpan ? block : kLaneSpan;
+  a.units = static_cast<int>((K + unit - 1) / unit);
   // Wavefronts per row (each owns whole units): four, which is also what staging the row uses,
   // eight for rows of sixteen units and more (measured: 5120 values in 5 units of 1024, 210 us on four
   // against 237 us on five; 13824 values in 27 units of 512, 608 us on eight against 655 us on four).

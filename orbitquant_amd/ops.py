@@ -95,6 +95,39 @@ def rotate_plan(permutation: torch.Tensor, signs: torch.Tensor, boundaries: torc
     return plan
 
 
+def quantize_weight(weight: torch.Tensor, permutation: torch.Tensor, signs: torch.Tensor, boundaries: torch.Tensor, *,
+                    bits: int, block_size: int, eps: float, inv_sqrt_block: float,
+                    row_tile: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """The weight side of a layer on the GPU (`oq_quantize_weight`): -> (packed uint8
+    [ceil(N*K*bits/8)], row_norms bfloat16 [N]) on the weight's device.  `row_tile` bounds the
+    rows converted per launch (the launches write disjoint byte ranges of the same stream, so the
+    result does not depend on it; tiles end on byte boundaries because K is a multiple of 8)."""
+    _require_gpu(weight, "weight")
+    if weight.ndim != 2:
+        raise ValueError("weight must be a matrix")
+    n, k = weight.shape
+    if weight.dtype not in _DTYPES:
+        raise ValueError(f"unsupported weight dtype {weight.dtype}")
+    w = weight.detach().contiguous()
+    permutation = _operand(permutation, "permutation", w, dtype=torch.int32, numel=k)
+    signs = _operand(signs, "signs", w, dtype=torch.int8, numel=k)
+    boundaries = _operand(boundaries, "boundaries", w, dtype=torch.float32)
+    plan = rotate_plan(permutation, signs, boundaries, block_size=block_size, inv_sqrt_block=inv_sqrt_block)
+    packed = torch.empty((n * k * bits + 7) // 8, dtype=torch.uint8, device=w.device)
+    norms = torch.empty(n, dtype=torch.bfloat16, device=w.device)
+    lib = _lib.load()
+    step = n if not row_tile else max(1, int(row_tile))
+    with _OnDevice(w):
+        for start in range(0, n, step):
+            rows = min(step, n - start)
+            rc = lib.oq_quantize_weight(
+                w.data_ptr() + start * k * w.element_size(), _dt(w), rows, k, plan.data_ptr(), boundaries.data_ptr(),
+                boundaries.numel() + 1, int(block_size), float(eps), float(inv_sqrt_block), int(bits),
+                packed.data_ptr() + start * k * bits // 8, norms.data_ptr() + 2 * start, _stream(w))
+            _lib.check(rc, "oq_quantize_weight")
+    return packed, norms
+
+
 def _plan_operand(plan: torch.Tensor | None, like: torch.Tensor, dim: int) -> torch.Tensor | None:
     if plan is None:
         return None
