@@ -275,10 +275,68 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
                             void *stream);
 
 /*
+ * Packed INT4 group-scaled linear on bf16 activations (the AdaLN modulation linears):
+ *
+ *   w[n,k]   = bf16( (q[n,k] - 8) * float(scales[n, k / group_size]) )
+ *   out[m,n] = bf16( sum_k x[m,k] * w[n,k] + float(bias[n]) )          (fp32 accumulation)
+ *
+ * Replaces matmul_packed_adaln_int4_cpu (torch_binding.cpp:47-66) and the reference's Triton
+ * kernel for it (src/orbitquant/kernels/triton_cuda.py:682-819) on AMD GPUs.
+ *
+ * x             bf16 [M, K] (raw bit patterns), row-major
+ * packed_weight 4-bit q, two per byte, low nibble first, rows padded to whole groups:
+ *               [N, groups * group_size / 2] bytes with groups = ceil(K / group_size)
+ *               (src/orbitquant/adaln.py:17-35)
+ * scales        bf16 [N, groups]
+ * bias          NULL or bf16 [N]
+ * out           bf16 [M, N]
+ * K a multiple of 8, group_size a multiple of 8 and a 16-byte aligned x take the streaming
+ * kernel, anything else a shape-agnostic one.
+ */
+int oq_matmul_packed_adaln_int4(const uint16_t *x, const uint8_t *packed_weight, const uint16_t *scales,
+                                const uint16_t *bias, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                                uint16_t *out, void *stream);
+
+/*
+ * The weight side of the AdaLN linears on the GPU: group-wise round-to-nearest INT4
+ * (src/orbitquant/adaln.py:17-35 `quantize_adaln_weight_int4`; the reference runs it as torch
+ * operations on whatever device holds the weight):
+ *
+ *   scale[n,g] = max(max_k |w[n,k]|, 1e-12) / 7            over the group's k, fp32, IEEE division
+ *   q[n,k]     = clamp(round_half_even(w[n,k] / scale[n,g]), -8, 7) + 8      (padding beyond K: 8)
+ *
+ * w          [N, K] of w_dtype (OQ_F32 / OQ_F16 / OQ_BF16), row-major
+ * packed_out [N * groups * group_size / 2] bytes, low nibble first, groups = ceil(K / group_size)
+ * scales_out fp32 [N, groups] (the module stores them rounded to bf16)
+ * group_size even.
+ */
+int oq_quantize_adaln_weight(const void *w, int w_dtype, int64_t N, int64_t K, int64_t group_size, uint8_t *packed_out,
+                             float *scales_out, void *stream);
+
+/*
  * Unpack a little-endian bit stream into one index per byte (debug / tests;
  * the GPU twin of unpack_lowbit, src/orbitquant/packing/bitpack.py:63-97).
  */
 int oq_unpack_lowbit(const uint8_t *packed, int bits, int64_t count, uint8_t *out, void *stream);
+
+/*
+ * The inverse of oq_unpack_lowbit: values[i] (its low `bits` bits) into bits [i * bits, (i + 1) * bits)
+ * of a little-endian stream of ceil(count * bits / 8) bytes, unused tail bits zero.
+ * Replaces pack_lowbit (src/orbitquant/packing/lowbit.py) and its Triton form
+ * (src/orbitquant/kernels/triton_cuda.py:878-899, 2681-2710) on AMD GPUs.  bits in [1, 8].
+ */
+int oq_pack_lowbit(const uint8_t *values, int bits, int64_t count, uint8_t *packed_out, void *stream);
+
+/*
+ * The dense form of a packed weight, in the rotated basis the layer multiplies in:
+ *   out[n,k] = centroids[index[n,k]] * float(row_norms[n])        (one fp32 product, then rounded to out_dtype)
+ * Replaces dequantize_packed_weight_with_triton (src/orbitquant/kernels/triton_cuda.py:523-547,
+ * 1538-1571; fp32 out there) for the reference's `dequant_bf16` debug mode.
+ * packed_weight  N * K indices of `bits` bits, one stream over the whole matrix
+ * row_norms      bf16 [N];  centroids fp32 [2^bits];  out [N, K] of out_dtype.
+ */
+int oq_dequantize_packed_weight(const uint8_t *packed_weight, int bits, const uint16_t *row_norms, const float *centroids,
+                                int64_t N, int64_t K, void *out, int out_dtype, void *stream);
 
 #ifdef __cplusplus
 }

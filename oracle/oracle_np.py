@@ -294,3 +294,45 @@ def matmul_packed_weight_f32(x32, packed, row_norms, centroids, bits, n, bias=No
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)[None, :]
     return y
+
+
+# --------------------------------------------------------------------------
+# AdaLN INT4 group-scaled linear
+# --------------------------------------------------------------------------
+
+def bf16_round(a: np.ndarray) -> np.ndarray:
+    """fp32 values rounded to bfloat16 (nearest even), returned as fp32."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=F32)).to(torch.bfloat16).float().numpy()
+
+
+def adaln_quantize(weight, group_size: int):
+    """src/orbitquant/adaln.py:17-35 - (packed u8, scales fp32 [N, groups], codes u8 [N, groups*group_size]).
+
+    Rows are zero-padded to whole groups; per group scale = max(absmax, 1e-12) / 7 in fp32,
+    code = clip(round_half_even(w / scale), -8, 7) + 8, two codes per byte, even index in the low nibble.
+    """
+    w = np.asarray(weight, dtype=F32)
+    n, k = w.shape
+    groups = (k + group_size - 1) // group_size
+    padded = np.zeros((n, groups * group_size), dtype=F32)
+    padded[:, :k] = w
+    grouped = padded.reshape(n, groups, group_size)
+    scales = (np.maximum(np.abs(grouped).max(axis=-1), F32(1e-12)) / F32(7.0)).astype(F32)
+    signed = np.clip(np.rint(grouped / scales[..., None]), -8, 7).astype(np.int16)
+    codes = (signed + 8).astype(np.uint8).reshape(n, groups * group_size)
+    flat = codes.reshape(-1)
+    packed = (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+    return packed, scales, codes
+
+
+def adaln_linear_f64(x, codes, scales_bf16, bias, in_features: int, group_size: int) -> np.ndarray:
+    """The contract of the packed AdaLN linear before its final rounding (adaln.py:300-312 dequantization,
+    cpu_msvc_avx2.cpp:186-236 of the reference): w = bf16((code - 8) * scale), y = x @ w.T + bias, here in fp64.
+    x: bf16-representable fp32 [M, K]; scales_bf16: the stored scales as fp32 [N, groups]; bias fp32 [N] or None."""
+    n = codes.shape[0]
+    signed = codes.astype(np.int16).astype(F32) - F32(8)
+    w = bf16_round((signed.reshape(n, -1, group_size) * np.asarray(scales_bf16, dtype=F32)[..., None]).reshape(n, -1))[:, :in_features]
+    y = np.asarray(x, dtype=np.float64) @ w.astype(np.float64).T
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)[None, :]
+    return y

@@ -2,7 +2,8 @@
 
 Public surface: `OrbitLinear`, `OrbitQuantConfig`, `recipe`, the host constants
 (`get_rpbh_rotation`, `get_codebook`, `pack_lowbit`, `unpack_lowbit`,
-`quantize_weight`) and `ops` (tensor wrappers over the C ABI).
+`quantize_weight`), `RTNInt4Linear` (the AdaLN INT4 linear), `load_artifact` / `save_artifact`
+(the reference's on-disk layout) and `ops` (tensor wrappers over the C ABI).
 """
 
 from .codebooks import LloydMaxCodebook, get_codebook
@@ -12,9 +13,11 @@ from .rotations import RPBHRotation, get_rpbh_rotation
 from .weights import quantize_weight
 from . import ops  # noqa: E402
 from .layers import OrbitLinear  # noqa: E402
+from .adaln import RTNInt4Linear, quantize_adaln_weight  # noqa: E402
+from .artifacts import load_artifact, save_artifact  # noqa: E402
 
 __all__ = [
-    "LloydMaxCodebook", "OrbitLinear", "OrbitQuantConfig", "RPBHRotation", "get_codebook",
-    "get_rpbh_rotation", "ops", "pack_lowbit", "packed_length", "quantize_weight", "recipe",
-    "unpack_lowbit",
+    "LloydMaxCodebook", "OrbitLinear", "OrbitQuantConfig", "RPBHRotation", "RTNInt4Linear", "get_codebook",
+    "get_rpbh_rotation", "load_artifact", "ops", "pack_lowbit", "packed_length", "quantize_adaln_weight",
+    "quantize_weight", "recipe", "save_artifact", "unpack_lowbit",
 ]

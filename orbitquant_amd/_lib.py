@@ -20,7 +20,8 @@ _STATUS = {1: "invalid argument", 2: "unsupported", 3: "launch failure"}
 
 EXPORTS = (
     "oq_device_ok", "oq_last_error", "oq_version", "oq_rotate_quantize", "oq_rotate_plan_bytes", "oq_rotate_plan_build", "oq_quantize_weight", "oq_rotate_quantize_mapped",
-    "oq_packed_linear", "oq_packed_linear_mapped", "oq_quantized_linear", "oq_quantized_linear_static", "oq_matmul_packed_weight", "oq_unpack_lowbit",
+    "oq_packed_linear", "oq_packed_linear_mapped", "oq_quantized_linear", "oq_quantized_linear_static", "oq_matmul_packed_weight", "oq_matmul_packed_adaln_int4", "oq_quantize_adaln_weight", "oq_unpack_lowbit", "oq_pack_lowbit",
+    "oq_dequantize_packed_weight",
 )
 
 _lib = None
@@ -71,6 +72,14 @@ def load() -> ctypes.CDLL:
     lib.oq_matmul_packed_weight.restype = c_int
     lib.oq_matmul_packed_weight.argtypes = [vp, c_int, vp, vp, c_int, vp, vp, vp, c_int,
                                             c_i64, c_i64, c_i64, vp, c_int, vp]
+    lib.oq_matmul_packed_adaln_int4.restype = c_int
+    lib.oq_matmul_packed_adaln_int4.argtypes = [vp, vp, vp, vp, c_i64, c_i64, c_i64, c_i64, vp, vp]
+    lib.oq_quantize_adaln_weight.restype = c_int
+    lib.oq_quantize_adaln_weight.argtypes = [vp, c_int, c_i64, c_i64, c_i64, vp, vp, vp]
+    lib.oq_pack_lowbit.restype = c_int
+    lib.oq_pack_lowbit.argtypes = [vp, c_int, c_i64, vp, vp]
+    lib.oq_dequantize_packed_weight.restype = c_int
+    lib.oq_dequantize_packed_weight.argtypes = [vp, c_int, vp, vp, c_i64, c_i64, vp, c_int, vp]
     lib.oq_unpack_lowbit.restype = c_int
     lib.oq_unpack_lowbit.argtypes = [vp, c_int, c_i64, vp, vp]
     _lib = lib

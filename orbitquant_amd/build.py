@@ -31,6 +31,8 @@ SOURCES = {
     "rotate_quantize.hip": ["-ffp-contract=off"],
     "rotate_quantize_fast.hip": ["-ffp-contract=off"],
     "packed_generic.hip": [],
+    "adaln_int4.hip": [],
+    "pack_utils.hip": [],
     "packed_gemm.hip": [],
     "packed_gemm_bytes.hip": [],
     "packed_gemm_av.hip": [],

@@ -24,6 +24,7 @@ class OrbitQuantConfig:
     activation_eps: float = 1e-10
     weight_row_tile_size: int = 256
     runtime_mode: str = "hip_packed"
+    adaln_group_size: int = 64
 
     def __post_init__(self) -> None:
         if self.weight_bits not in SUPPORTED_BITS:
@@ -34,6 +35,8 @@ class OrbitQuantConfig:
             raise ValueError("only codebook_version 2 is implemented")
         if self.block_size != "paper" and (not isinstance(self.block_size, int) or self.block_size <= 0):
             raise ValueError("block_size must be 'paper' or a positive int")
+        if self.adaln_group_size <= 0:
+            raise ValueError("adaln_group_size must be positive")
         if self.activation_eps <= 0:
             raise ValueError("activation_eps must be positive")
         if self.runtime_mode not in {"hip_packed", "auto_fused", "native_packed_matmul"}:

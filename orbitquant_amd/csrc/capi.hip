@@ -70,6 +70,13 @@ int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *bou
 int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,
                          int levels, int64_t block, float eps, float inv_sqrt_block, int bits, uint8_t *packed_out,
                          uint16_t *row_norms_out, hipStream_t stream);
+int adaln_int4_dispatch(const uint16_t *x, const uint8_t *packed, const uint16_t *scales, const uint16_t *bias, int64_t M,
+                        int64_t N, int64_t K, int64_t group, uint16_t *out, hipStream_t stream);
+int adaln_quantize_dispatch(const void *w, int w_dtype, int64_t N, int64_t K, int64_t group, uint8_t *packed, float *scales,
+                            hipStream_t stream);
+int pack_lowbit_dispatch(const uint8_t *values, int bits, int64_t count, uint8_t *packed, hipStream_t stream);
+int dequantize_dispatch(const uint8_t *packed, int bits, const uint16_t *row_norms, const float *centroids, int64_t N, int64_t K,
+                        void *out, int out_dtype, hipStream_t stream);
 bool token_linear_supported(int x_dtype, int64_t M, int64_t N, int64_t K, int levels, int bits, const void *x,
                             const int32_t *perm, const int8_t *signs);
 int token_linear_dispatch(const void *x, int x_dtype, const uint16_t *input_map, int64_t K, const int32_t *perm,
@@ -331,10 +338,36 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
                               K, out, out_dtype, s);
 }
 
+int oq_matmul_packed_adaln_int4(const uint16_t *x, const uint8_t *packed_weight, const uint16_t *scales,
+                                const uint16_t *bias, int64_t M, int64_t N, int64_t K, int64_t group_size, uint16_t *out,
+                                void *stream) {
+  return adaln_int4_dispatch(x, packed_weight, scales, bias, M, N, K, group_size, out, as_stream(stream));
+}
+
+int oq_quantize_adaln_weight(const void *w, int w_dtype, int64_t N, int64_t K, int64_t group_size, uint8_t *packed_out,
+                             float *scales_out, void *stream) {
+  return adaln_quantize_dispatch(w, w_dtype, N, K, group_size, packed_out, scales_out, as_stream(stream));
+}
+
 int oq_unpack_lowbit(const uint8_t *packed, int bits, int64_t count, uint8_t *out, void *stream) {
   if (bits < 1 || bits > 8 || count < 0) return fail(OQ_ERR_INVALID, "unpack_lowbit: bits=%d count=%lld", bits, (long long)count);
   if (count > 0 && (packed == nullptr || out == nullptr)) return fail(OQ_ERR_INVALID, "unpack_lowbit: null pointer");
   return unpack_dispatch(packed, bits, count, out, as_stream(stream));
+}
+
+int oq_pack_lowbit(const uint8_t *values, int bits, int64_t count, uint8_t *packed_out, void *stream) {
+  if (bits < 1 || bits > 8 || count < 0) return fail(OQ_ERR_INVALID, "pack_lowbit: bits=%d count=%lld", bits, (long long)count);
+  if (count > 0 && (values == nullptr || packed_out == nullptr)) return fail(OQ_ERR_INVALID, "pack_lowbit: null pointer");
+  return pack_lowbit_dispatch(values, bits, count, packed_out, as_stream(stream));
+}
+
+int oq_dequantize_packed_weight(const uint8_t *packed_weight, int bits, const uint16_t *row_norms, const float *centroids,
+                                int64_t N, int64_t K, void *out, int out_dtype, void *stream) {
+  if (bits < 1 || bits > 8 || N < 0 || K < 0) return fail(OQ_ERR_INVALID, "dequantize_packed_weight: bits=%d N=%lld K=%lld", bits, (long long)N, (long long)K);
+  if (out_dtype != OQ_F32 && out_dtype != OQ_F16 && out_dtype != OQ_BF16) return fail(OQ_ERR_INVALID, "dequantize_packed_weight: out_dtype=%d", out_dtype);
+  if (N > 0 && K > 0 && (packed_weight == nullptr || row_norms == nullptr || centroids == nullptr || out == nullptr))
+    return fail(OQ_ERR_INVALID, "dequantize_packed_weight: null pointer");
+  return dequantize_dispatch(packed_weight, bits, row_norms, centroids, N, K, out, out_dtype, as_stream(stream));
 }
 
 }  // extern "C"

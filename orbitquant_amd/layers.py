@@ -196,6 +196,21 @@ class OrbitLinear(nn.Module):
             module_name=module_name)
 
     @classmethod
+    def empty_from_linear(cls, layer: nn.Linear, *, config: OrbitQuantConfig, module_name: str = "") -> "OrbitLinear":
+        """A skeleton with the right tensor shapes for a packed state dict to be loaded into
+        (src/orbitquant/layers.py:510-561 of the reference); the constants (rotation, codebooks,
+        rotate plan) are those of (in_features, config) already."""
+        if not isinstance(layer, nn.Linear):
+            raise TypeError(f"no OrbitQuant linear adapter registered for {type(layer).__name__}")
+        n, k = layer.out_features, layer.in_features
+        device = layer.weight.device
+        bias = None if layer.bias is None else torch.zeros(n, dtype=layer.bias.dtype, device=device)
+        return cls(
+            in_features=k, out_features=n, config=config, bias=bias,
+            packed_weight_indices=torch.zeros(packed_length(n * k, config.weight_bits), dtype=torch.uint8, device=device),
+            row_norms=torch.zeros(n, dtype=torch.bfloat16, device=device), module_name=module_name)
+
+    @classmethod
     def from_linear(cls, layer: nn.Linear, *, config: OrbitQuantConfig, module_name: str = "") -> "OrbitLinear":
         if not isinstance(layer, nn.Linear):
             raise TypeError(f"no OrbitQuant linear adapter registered for {type(layer).__name__}")

@@ -383,6 +383,88 @@ def matmul_packed_weight_values(
     return out.reshape(*lead, out_features)
 
 
+def adaln_int4_linear(x: torch.Tensor, packed_weight: torch.Tensor, scales: torch.Tensor, *, out_features: int,
+                      in_features: int, group_size: int, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """The packed INT4 group-scaled linear of the AdaLN modules (`oq_matmul_packed_adaln_int4`):
+    x is taken as bfloat16, the result is bfloat16 (as the reference's kernels for it)."""
+    _require_gpu(x, "x")
+    if x.shape[-1] != in_features:
+        raise ValueError(f"expected input last dimension {in_features}, got {x.shape[-1]}")
+    if group_size <= 0:
+        raise ValueError("group_size must be positive")
+    lead = x.shape[:-1]
+    flat = x.to(torch.bfloat16).contiguous().reshape(-1, in_features)
+    m = flat.shape[0]
+    groups = (in_features + group_size - 1) // group_size
+    packed_weight = _operand(packed_weight, "packed_weight", flat, dtype=torch.uint8,
+                             numel=(out_features * groups * group_size * 4 + 7) // 8)
+    scales = _operand(scales, "scales", flat, dtype=torch.bfloat16, numel=out_features * groups)
+    if bias is not None and bias.dtype != torch.bfloat16:
+        bias = bias.to(torch.bfloat16)
+    bias = _operand(bias, "bias", flat, dtype=torch.bfloat16, numel=out_features)
+    out = torch.empty((m, out_features), dtype=torch.bfloat16, device=flat.device)
+    lib = _lib.load()
+    with _OnDevice(flat):
+        rc = lib.oq_matmul_packed_adaln_int4(flat.data_ptr(), packed_weight.data_ptr(), scales.data_ptr(), _ptr(bias), m,
+                                             int(out_features), int(in_features), int(group_size), out.data_ptr(), _stream(flat))
+    _lib.check(rc, "oq_matmul_packed_adaln_int4")
+    return out.reshape(*lead, out_features)
+
+
+def quantize_adaln_weight(weight: torch.Tensor, *, group_size: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Group-wise round-to-nearest INT4 of a weight on the GPU (`oq_quantize_adaln_weight`):
+    -> (packed uint8 [N * groups * group_size / 2], scales float32 [N, groups])."""
+    _require_gpu(weight, "weight")
+    if weight.ndim != 2 or weight.dtype not in _DTYPES:
+        raise ValueError("weight must be a float32/float16/bfloat16 matrix")
+    if group_size <= 0 or group_size % 2:
+        raise ValueError("the GPU quantizer takes even group sizes")
+    weight = weight.contiguous()
+    n, k = weight.shape
+    groups = (k + group_size - 1) // group_size
+    packed = torch.empty(n * groups * group_size // 2, dtype=torch.uint8, device=weight.device)
+    scales = torch.empty(n, groups, dtype=torch.float32, device=weight.device)
+    lib = _lib.load()
+    with _OnDevice(weight):
+        rc = lib.oq_quantize_adaln_weight(weight.data_ptr(), _DTYPES[weight.dtype], n, k, int(group_size), packed.data_ptr(),
+                                          scales.data_ptr(), _stream(weight))
+    _lib.check(rc, "oq_quantize_adaln_weight")
+    return packed, scales
+
+
+def pack_lowbit(values: torch.Tensor, bits: int) -> torch.Tensor:
+    """uint8 indices -> the little-endian `bits`-wide stream (`oq_pack_lowbit`)."""
+    _require_gpu(values, "values")
+    values = _operand(values.reshape(-1), "values", values, dtype=torch.uint8)
+    count = values.numel()
+    packed = torch.empty((count * int(bits) + 7) // 8, dtype=torch.uint8, device=values.device)
+    lib = _lib.load()
+    with _OnDevice(values):
+        rc = lib.oq_pack_lowbit(values.data_ptr(), int(bits), count, packed.data_ptr(), _stream(values))
+    _lib.check(rc, "oq_pack_lowbit")
+    return packed
+
+
+def dequantize_packed_weight(packed_weight: torch.Tensor, row_norms: torch.Tensor, centroids: torch.Tensor, *, bits: int,
+                             out_features: int, in_features: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """centroids[index] * row_norm as a dense [out_features, in_features] matrix in the rotated
+    basis (`oq_dequantize_packed_weight`)."""
+    _require_gpu(packed_weight, "packed_weight")
+    if dtype not in _DTYPES:
+        raise ValueError(f"dtype must be one of {_FLOATS}")
+    total = int(out_features) * int(in_features)
+    packed_weight = _operand(packed_weight, "packed_weight", packed_weight, dtype=torch.uint8, min_numel=(total * int(bits) + 7) // 8)
+    row_norms = _operand(row_norms, "row_norms", packed_weight, dtype=torch.bfloat16, numel=out_features)
+    centroids = _operand(centroids, "centroids", packed_weight, dtype=torch.float32, numel=1 << int(bits))
+    out = torch.empty(out_features, in_features, dtype=dtype, device=packed_weight.device)
+    lib = _lib.load()
+    with _OnDevice(packed_weight):
+        rc = lib.oq_dequantize_packed_weight(packed_weight.data_ptr(), int(bits), row_norms.data_ptr(), centroids.data_ptr(),
+                                             int(out_features), int(in_features), out.data_ptr(), _DTYPES[dtype], _stream(packed_weight))
+    _lib.check(rc, "oq_dequantize_packed_weight")
+    return out
+
+
 def unpack_lowbit(packed: torch.Tensor, bits: int, length: int) -> torch.Tensor:
     _require_gpu(packed, "packed")
     packed = _operand(packed, "packed", packed, dtype=torch.uint8, min_numel=(int(length) * int(bits) + 7) // 8)

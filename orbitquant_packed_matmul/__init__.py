@@ -68,6 +68,21 @@ def matmul_packed_adaln_int4_cpu(*args, **kwargs):
     raise RuntimeError("this build of orbitquant_packed_matmul has no CPU kernels (AMD GPU only)")
 
 
+def matmul_packed_adaln_int4(x, packed_weight, scales, *, out_features, in_features, group_size, bias=None):
+    """The AMD GPU form of `matmul_packed_adaln_int4_cpu` (same arguments and result, torch-ext
+    `__init__.py`:163-204 of the reference): bf16 activations times the packed INT4 group-scaled
+    weight, bf16 out."""
+    from orbitquant_amd import ops
+
+    if x.device.type != "cuda":
+        raise RuntimeError("native packed AdaLN requires AMD GPU tensors (torch device 'cuda')")
+    device = x.device
+    return ops.adaln_int4_linear(
+        x, packed_weight.to(device=device, dtype=torch.uint8), scales.to(device=device, dtype=torch.bfloat16),
+        out_features=out_features, in_features=in_features, group_size=group_size,
+        bias=None if bias is None else bias.to(device=device, dtype=torch.bfloat16))
+
+
 def matmul_packed_weight(
     x: torch.Tensor,
     packed_weight_indices: torch.Tensor,
