@@ -453,6 +453,40 @@ def c3_gemm_lines(device, iters):
     return out
 
 
+def float_activation_lines(device, iters):
+    """`oq_matmul_packed_weight` (bf16 activation values times the packed weight, the reference's generic
+    contract) on the two c2 shapes: the whole call, i.e. the pass that puts the activations into operand
+    order plus the tile kernel, timed with events over back-to-back eager calls."""
+    from orbitquant_amd import ops
+
+    spec = workload_spec("c2", 0)
+    gen = torch.Generator().manual_seed(9)
+    layers = build_layers(spec, device, gen, False)
+    out = {}
+    for layer, _act in layers:
+        k, n = layer.in_features, layer.out_features
+        x = make_input(spec, k, gen).to(device)
+        cents = layer._weight_codebook_centroids
+
+        def fn():
+            ops.matmul_packed_weight_values(x, layer.packed_weight_indices, layer.row_norms, cents, bits=layer.weight_bits,
+                                            out_features=n, in_features=k)
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = max(20, iters)
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        t = start.elapsed_time(stop) / reps * 1e-3
+        tflops = 2.0 * spec["M"] * n * k / t / 1e12
+        out[f"{k}->{n}"] = {"call_us": t * 1e6, "tflops": tflops, "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
+    return out
+
+
 def build_c5(device, gen):
     """The 240 distinct matrices of the 40-layer decode stack: per layer q,k (4096x4096), v,o
     (4096x4096), up (14336x4096), down (4096x14336); interior layers q,k W2 and the rest W3,
@@ -658,6 +692,7 @@ def main() -> int:
         # the two other figures the metric names, each on its own roofline kernel (`--workload c3|c5` for the full runs)
         out["roofline_small_m"] = small_m_roofline(device, args.kernel_iters)
         out["c3_gemms"] = c3_gemm_lines(device, args.kernel_iters)
+        out["float_activations"] = float_activation_lines(device, args.kernel_iters)
     copy_calibration(device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, layers, x)

@@ -35,6 +35,7 @@ SOURCES = {
     "pack_utils.hip": [],
     "packed_gemm.hip": [],
     "packed_gemm_bytes.hip": [],
+    "packed_gemm_tiled.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
     "token_linear.hip": [],

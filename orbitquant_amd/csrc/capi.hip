@@ -70,6 +70,9 @@ int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *bou
 int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,
                          int levels, int64_t block, float eps, float inv_sqrt_block, int bits, uint8_t *packed_out,
                          uint16_t *row_norms_out, hipStream_t stream);
+int gemm_tiled_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
+                        const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
+                        int out_dtype, hipStream_t stream);
 int adaln_int4_dispatch(const uint16_t *x, const uint8_t *packed, const uint16_t *scales, const uint16_t *bias, int64_t M,
                         int64_t N, int64_t K, int64_t group, uint16_t *out, hipStream_t stream);
 int adaln_quantize_dispatch(const void *w, int w_dtype, int64_t N, int64_t K, int64_t group, uint8_t *packed, float *scales,
@@ -325,6 +328,16 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   if (M == 0) return OQ_OK;
   if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
   hipStream_t s = as_stream(stream);
+  if (x_dtype == OQ_BF16 && M >= 256 && K % 64 == 0 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) &&
+      gemm_supported(K, bits)) {
+    // Large M: one pass puts the activations into the matrix core's operand order, then the tile kernel runs on them
+    // (not while the stream is being captured into a graph: the pass needs memory).
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
+      const int rc = gemm_tiled_dispatch(x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+      if (rc >= 0) return rc;
+    }
+  }
   if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
   {
     // The float-activation kernel has its own (measured) preference: 256x256 tiles once there are

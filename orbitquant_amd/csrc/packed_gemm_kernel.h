@@ -41,10 +41,15 @@
 
 namespace oq {
 
-enum AMode { A_NIBBLE = 0, A_U8 = 1 };  // activation codes: two per byte, or one per byte
+// Activations: codes two per byte, codes one per byte, or 16-bit values (bf16) already in the matrix
+// core's operand order: 16-byte piece ((row_tile * K/64 + k_step) * 4 + q) * 64 + lane holds, for lane
+// (r = lane % 32, g = lane / 32), the eight values k_step*64 + 32g + 8q .. +7 of row 32*row_tile + r
+// (tile_activations_kernel writes it).  Then a wavefront's activation load is 1 KB of consecutive
+// bytes, the operand needs no lookup, and only the weights go through the tables.
+enum AMode { A_NIBBLE = 0, A_U8 = 1, A_TILED = 2 };
 
 struct GemmArgs {
-  const uint8_t *a;          // [M, K/2] nibble codes or [M, K] one code per byte
+  const uint8_t *a;          // [M, K/2] nibble codes, [M, K] one code per byte, or the tiled 16-bit values
   const float *row_scale;    // [M] or NULL
   const float *act_cents;    // [a_levels]
   int a_levels;
@@ -85,7 +90,9 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // are written while the packed data is still in flight.
   const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
   uint32_t my_a;
-  if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
+  if constexpr (AM == A_TILED) {
+    my_a = 0u;                     // no activation table
+  } else if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
     const int c0 = tid & 15, c1 = tid >> 4;
     my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
   } else {                         // row = one code, its value in both halves of the dword
@@ -116,14 +123,18 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   EpiFactors<FM> epi;
   gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
 
-  constexpr int kAStep = AM == A_NIBBLE ? 32 : 64;  // bytes of one activation row per K-step of 64
-  constexpr int kAVec = kAStep / 32;                // 16-byte loads per lane per K-step
+  constexpr int kAStep = AM == A_NIBBLE ? 32 : AM == A_U8 ? 64 : 4096;  // bytes from one K-step of 64 to the next in a lane's activation stream
+  constexpr int kAVec = AM == A_NIBBLE ? 1 : AM == A_U8 ? 2 : 4;        // 16-byte loads per lane per K-step
+  constexpr int kAVecStride = AM == A_TILED ? 1024 : 16;
   const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K;
   const int64_t w_row_bytes = g.K * BITS / 8;
   const uint8_t *ap[FM];
   const uint8_t *wp[FN];
 #pragma unroll
-  for (int i = 0; i < FM; ++i) ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
+  for (int i = 0; i < FM; ++i) {
+    if constexpr (AM == A_TILED) ap[i] = g.a + min(m_base / 32 + i, (g.M + 31) / 32 - 1) * (g.K / 64) * kAStep + lane * 16;
+    else ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
+  }
 #pragma unroll
   for (int j = 0; j < FN; ++j) wp[j] = g.w + min(n_base + 32 * j + r, g.N - 1) * w_row_bytes + grp * (4 * BITS);
 
@@ -143,7 +154,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     const int64_t s = min(ks, steps - 1);  // past the end: re-read the last step (never multiplied)
     if (e < FM) {
 #pragma unroll
-      for (int v = 0; v < kAVec; ++v) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + 16 * v);
+      for (int v = 0; v < kAVec; ++v) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + kAVecStride * v);
     }
     else load_w<BITS>(wp[e - FM] + s * (8 * BITS), pw[B][e - FM]);
   };
@@ -176,10 +187,11 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   //
   // One-code-per-byte activations take two lookups per operand dword (single-code table, the
   // value in both halves); the two are merged with one v_perm_b32 when the operand is used.
-  constexpr int kRA = AM == A_NIBBLE ? 4 : 8;  // LDS reads per activation tile and phase
+  constexpr int kRA = AM == A_NIBBLE ? 4 : AM == A_U8 ? 8 : 0;  // LDS reads per activation tile and phase
+  constexpr int kRAd = kRA > 0 ? kRA : 1;
   constexpr int kLookups = kRA * FM + 4 * FN, kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
   constexpr int kLook = (kLookups + kGroups - 1) / kGroups;
-  uint32_t oa[2][FM][kRA], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
+  uint32_t oa[2][FM][kRAd], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
 
   // dword d (0..7 for bytes, 0..3 for nibbles) of this lane's activation run in buffer B, tile i
   auto a_word = [&](auto buf, int i, int d) -> uint32_t {
@@ -193,11 +205,13 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   auto lookup_address = [&](auto buf, int q, int t) -> uint32_t {
     constexpr int B = decltype(buf)::value;
     const bool is_a = t < kRA || t >= kRA + 4 * FN;
-    if (is_a) {
-      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
-      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
-      if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
-      else return row_address(a_word(buf, i, 2 * q + (sub >> 2)), a_off, sub & 3);  // byte 8q + sub of the run
+    if constexpr (kRA > 0) {
+      if (is_a) {
+        const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRAd;
+        const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRAd;
+        if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
+        else return row_address(a_word(buf, i, 2 * q + (sub >> 2)), a_off, sub & 3);  // byte 8q + sub of the run
+      }
     }
     const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
     if constexpr (BITS == 4) return row_address(pw[B][j][q], w_off, p);
@@ -205,10 +219,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   };
   auto lookup_read = [&](auto buf, int q, int set, int t, uint32_t address) {
     constexpr int B = decltype(buf)::value;
-    const bool is_a = t < kRA || t >= kRA + 4 * FN;
+    const bool is_a = kRA > 0 && (t < kRA || t >= kRA + 4 * FN);
     if (is_a) {
-      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRA;
-      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRA;
+      const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRAd;
+      const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRAd;
       oa[set][i][sub] = lds_read_u32(address);
     } else {
       const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
@@ -218,7 +232,9 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   };
   // the activation operand of tile i out of `set`
   auto a_operand = [&](int set, int i) -> uint4 {
-    if constexpr (AM == A_NIBBLE) {
+    if constexpr (AM == A_TILED) {
+      return make_uint4(0u, 0u, 0u, 0u);  // (the operand comes straight from the load registers, see phase)
+    } else if constexpr (AM == A_NIBBLE) {
       return make_uint4(oa[set][i][0], oa[set][i][1], oa[set][i][2], oa[set][i][3]);
     } else {
       return make_uint4(__builtin_amdgcn_perm(oa[set][i][1], oa[set][i][0], 0x07060100u),
@@ -228,7 +244,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     }
   };
   // lookups of (buf, q) into `set` interleaved with the MFMAs on the other set
-  auto phase = [&](auto buf, int q, int set, auto fetch_buf, int fetch_ks, bool with_fetch) {
+  // (mul_buf, mul_q): the K-step buffer and MFMA index of the operands being multiplied, i.e. of the previous phase
+  auto phase = [&](auto buf, int q, int set, auto fetch_buf, int fetch_ks, bool with_fetch, auto mul_buf, auto mul_q) {
     uint32_t addr[2][kLook];
     uint4 av = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
@@ -236,7 +253,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #pragma unroll
     for (int m = 0; m < kGroups; ++m) {
       const int i = m / FN, j = m % FN;
-      if (j == 0) av = a_operand(set ^ 1, i);
+      if (j == 0) {
+        if constexpr (AM == A_TILED) av = pa[decltype(mul_buf)::value][i][decltype(mul_q)::value];
+        else av = a_operand(set ^ 1, i);
+      }
       const int lo = m * kLookups / kGroups, hi = (m + 1) * kLookups / kGroups, hi2 = (m + 2) * kLookups / kGroups;
       if (with_fetch && m < FM + FN) fetch_one(fetch_buf, m, fetch_ks);
       const uint4 bw = make_uint4(ob[set ^ 1][j][0], ob[set ^ 1][j][1], ob[set ^ 1][j][2], ob[set ^ 1][j][3]);
@@ -257,11 +277,11 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     constexpr int B = decltype(buf)::value;
     constexpr auto prev = std::integral_constant<int, (B + NBUF - 1) % NBUF>{};
     constexpr auto next = std::integral_constant<int, (B + 1) % NBUF>{};
-    phase(buf, 1, 1, prev, ks + NBUF - 1, FM + FN <= FM * FN);
+    phase(buf, 1, 1, prev, ks + NBUF - 1, FM + FN <= FM * FN, buf, std::integral_constant<int, 0>{});
     if constexpr (FM + FN > FM * FN) fetch(prev, ks + NBUF - 1);
-    phase(buf, 2, 0, prev, 0, false);
-    phase(buf, 3, 1, prev, 0, false);
-    phase(next, 0, 0, prev, 0, false);
+    phase(buf, 2, 0, prev, 0, false, buf, std::integral_constant<int, 1>{});
+    phase(buf, 3, 1, prev, 0, false, buf, std::integral_constant<int, 2>{});
+    phase(next, 0, 0, prev, 0, false, buf, std::integral_constant<int, 3>{});
   };
 
 #pragma unroll

@@ -582,3 +582,32 @@ def test_dropin_matmul_packed_weight_rows_1536(dev):
         want = o.matmul_packed_weight_f32(x.float().numpy(), layer["packed"], layer["r"].float().numpy(), layer["cw"], 4, 1536)
         s = np.linalg.norm(x.float().numpy(), axis=1)
         check_outputs(got, want, s, layer["r"].float().numpy(), 1536, f"rows {rows}")
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
+@pytest.mark.parametrize(("m", "n", "k"), [(300, 200, 256), (512, 1152, 4608), (257, 96, 64), (2048, 384, 1152)])
+def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k):
+    """bf16 activations at M >= 256 take the operand-order pass + tile kernel: against the oracle, and
+    bit for bit against the code kernel fed with the codes whose centroids are those activations."""
+    from orbitquant_amd import ops
+
+    rng = np.random.default_rng(bits * 7 + m)
+    layer = make_layer(rng, n, k, bits, 4)
+    ca = torch.from_numpy(layer["ca"]).to(torch.bfloat16)             # sixteen bf16 values
+    codes = rng.integers(0, 16, size=(m, k), dtype=np.uint8)
+    x = ca[torch.from_numpy(codes).long()] if m != 300 else torch.from_numpy(rng.standard_normal((m, k)).astype(F32)).to(torch.bfloat16)
+    scale = torch.from_numpy(rng.uniform(0.5, 2.0, m).astype(F32))
+    bias = torch.from_numpy(layer["bias"]).to(torch.bfloat16)
+    args = dict(bits=bits, out_features=n, in_features=k, bias=bias.to(dev), token_scale=scale.to(dev))
+    got = ops.matmul_packed_weight_values(x.to(dev), torch.from_numpy(layer["packed"]).to(dev), layer["r"].to(dev),
+                                          torch.from_numpy(layer["cw"]).to(dev), **args)
+    want = o.matmul_packed_weight_f32(x.float().numpy(), layer["packed"], layer["r"].float().numpy(), layer["cw"], bits, n, None)
+    want = want * scale.numpy()[:, None] + bias.float().numpy()[None, :]
+    s = np.linalg.norm(x.float().numpy(), axis=1) * scale.numpy()
+    check_outputs(got, want, s, layer["r"].float().numpy(), k, f"large-M float activations W{bits}")
+    if m != 300:
+        nib = torch.from_numpy((codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8))
+        by_codes = ops.packed_linear(nib.to(dev), scale.to(dev), torch.from_numpy(layer["ca"]).to(dev), torch.from_numpy(layer["packed"]).to(dev),
+                                     layer["r"].to(dev), torch.from_numpy(layer["cw"]).to(dev), code_format="nibble", activation_bits=4,
+                                     weight_bits=bits, out_features=n, in_features=k, bias=bias.to(dev), output_dtype=torch.bfloat16)
+        assert torch.equal(got, by_codes)
