@@ -35,6 +35,8 @@ def parse_args():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--m", type=int, default=0, help="token count override (c5: 1, 4 or 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-shared-quantization", action="store_true",
+                    help="c5: q, k and v each quantize their (common) input, as the reference's layers do")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
     ap.add_argument("--kernel-iters", type=int, default=50)
     ap.add_argument("--activation", default="output", choices=["output", "input", "separate"],
@@ -513,12 +515,19 @@ def bench_c5(args, device):
     gen = torch.Generator().manual_seed(5)
     m = args.m or 1
     mats = build_c5(device, gen)
-    x4096 = torch.randn(m, 4096, generator=gen).to(torch.bfloat16).to(device)
+    # one input per role, as in a transformer block: q, k and v read the same tensor (and share its
+    # quantization, `share_input_quantization`), o, up and down each their own
+    x_attn, x_o, x_up = (torch.randn(m, 4096, generator=gen).to(torch.bfloat16).to(device) for _ in range(3))
     x14336 = torch.randn(m, 14336, generator=gen).to(torch.bfloat16).to(device)
+    roles = ("q", "k", "v", "o", "up", "down")
+    inputs = {"q": x_attn, "k": x_attn, "v": x_attn, "o": x_o, "up": x_up, "down": x14336}
+    layer_input = [inputs[roles[i % 6]] for i in range(len(mats))]
+    if not args.no_shared_quantization:
+        for i, l in enumerate(mats):
+            l.share_input_quantization = roles[i % 6] in ("q", "k", "v")
     packed_bytes = sum(l.packed_weight_indices.numel() + 2 * l.out_features for l in mats)
     pre = []
-    for l in mats:
-        x = x4096 if l.in_features == 4096 else x14336
+    for l, x in zip(mats, layer_input):
         codes, _, norms = ops.rotate_quantize(
             x, l._rotation_permutation, l._rotation_signs, l._activation_codebook_boundaries,
             block_size=l.rotation.block_size, eps=l.activation_eps, inv_sqrt_block=l.rotation.normalization,
@@ -533,13 +542,13 @@ def bench_c5(args, device):
                               output_dtype=torch.bfloat16)
 
     def full_step():
-        for l in mats:
-            l(x4096 if l.in_features == 4096 else x14336)
+        for l, x in zip(mats, layer_input):
+            l(x)
 
     def full_step_out():
         last = None
-        for l in mats:
-            last = l(x4096 if l.in_features == 4096 else x14336)
+        for l, x in zip(mats, layer_input):
+            last = l(x)
         return last
 
     preroll(full_step)
@@ -558,8 +567,7 @@ def bench_c5(args, device):
     lib = _lib.load()
     stream = torch.cuda.current_stream(device).cuda_stream
     keep, calls = [], []
-    for l in mats:
-        x = x4096 if l.in_features == 4096 else x14336
+    for l, x in zip(mats, layer_input):
         nib = l.in_features // 2
         bufs = (torch.empty((m, nib), dtype=torch.uint8, device=device), torch.empty(m, dtype=torch.float32, device=device),
                 torch.empty((m, l.out_features), dtype=torch.bfloat16, device=device))
@@ -578,7 +586,7 @@ def bench_c5(args, device):
                 raise RuntimeError(lib.oq_last_error().decode())
     abi_step()
     torch.cuda.synchronize()
-    assert torch.equal(keep[-1][2], mats[-1](x14336)), "C-ABI stack differs from the module stack"
+    assert torch.equal(keep[-1][2], mats[-1](x14336)) and torch.equal(keep[2][2], mats[2](x_attn)), "C-ABI stack differs from the module stack"
     abi_dt = time_steps(abi_step, args.steps, args.warmup)
 
     # kernel-only: every matmul launch of the stack, events on the launch stream
@@ -600,6 +608,7 @@ def bench_c5(args, device):
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "config": {"workload": f"c5 40-layer decode stack W2/W3/W4 A4, M={m}", "M": m,
                                         "packed_bytes_per_step": packed_bytes, "launch": launch,
+                                        "shared_quantization": "none" if args.no_shared_quantization else "q, k, v of a block quantize their common input once",
                                         "eager_ms_per_step": eager_dt * 1e3,
                                         "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
                                         "c_abi_ms_per_step": abi_dt * 1e3,

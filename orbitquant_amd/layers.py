@@ -89,6 +89,9 @@ def packed_length(value_count: int, bits: int) -> int:
     return (value_count * bits + 7) // 8
 
 
+_last_quantization: dict = {}  # the one entry of OrbitLinear._forward_shared
+
+
 class OrbitLinear(nn.Module):
     def __init__(
         self,
@@ -132,6 +135,10 @@ class OrbitLinear(nn.Module):
         self.register_buffer("_input_activation_table", None, persistent=False)
         self._output_activation = None
         self.register_buffer("_output_activation_table", None, persistent=False)
+        # Linears that read the same tensor (q, k and v of an attention block; gate and up of an MLP) can
+        # share its quantization: set this on each of them and the codes the first one computes serve the
+        # others (see _shared_codes).  Off by default: the reference quantizes per layer.
+        self.share_input_quantization = False
 
     def fuse_input_activation(self, fn, *, dtype: torch.dtype = torch.bfloat16) -> "OrbitLinear":
         """Make forward(x) return what forward(fn(x)) returns, bit for bit, without a separate
@@ -245,12 +252,42 @@ class OrbitLinear(nn.Module):
         if out_table is not None and out_table.dtype != x.dtype:
             raise ValueError(f"the fused output activation was built for {out_table.dtype}, got {x.dtype}")
         self.last_effective_runtime_mode = "hip_packed"
+        if self.share_input_quantization and not torch.compiler.is_compiling():
+            return self._forward_shared(x, table, out_table)
         return torch.ops.orbitquant_amd.quantized_linear(
             x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_centroids,
             self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
             self._weight_codebook_centroids, self.bias, self.rotation.block_size,
             self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
             self.out_features, table, out_table, self._rotation_plan)
+
+    def _forward_shared(self, x, table, out_table):
+        """The forward as quantize + packed linear, with the codes of the most recent quantization kept
+        (one entry, process-wide): a layer whose input is the same tensor, unchanged (same storage
+        address, shape, dtype and version counter), quantized by the same rotation and codebook, skips
+        its quantizer.  Same kernels as the fused op, so the same output bits.  The entry holds a
+        reference to the input, so its address cannot be handed to another tensor meanwhile; writes
+        to the input that bypass torch's version counter are not seen."""
+        fmt = "nibble" if self.activation_bits <= 4 else "u8"
+        key = (x.data_ptr(), x._version, tuple(x.shape), x.dtype, x.device, self.in_features, self.rotation.seed,
+               self.rotation.block_size, self.activation_bits, self.activation_eps,
+               None if table is None else table.data_ptr())
+        entry = _last_quantization
+        if entry.get("key") == key:
+            codes, norms = entry["codes"], entry["norms"]
+        else:
+            codes, _, norms = ops.rotate_quantize(
+                x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_boundaries,
+                block_size=self.rotation.block_size, eps=self.activation_eps, inv_sqrt_block=self.rotation.normalization,
+                code_format=fmt, input_map=table, plan=self._rotation_plan)
+            entry.update(key=key, codes=codes, norms=norms, keep=x)
+        bias = self.bias
+        if bias is not None and bias.dtype != x.dtype:
+            bias = bias.to(x.dtype)   # as the fused op (and the reference on accelerators) does
+        return ops.packed_linear(codes, norms, self._activation_codebook_centroids, self.packed_weight_indices, self.row_norms,
+                                 self._weight_codebook_centroids, code_format=fmt, activation_bits=self.activation_bits,
+                                 weight_bits=self.weight_bits, out_features=self.out_features, in_features=self.in_features,
+                                 bias=bias, output_dtype=x.dtype, output_map=out_table)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

@@ -145,3 +145,38 @@ def test_layer_forward_one_token_matches_batched_rows(dev):
     assert (batched - single).abs().max().item() <= 2e-2 * scale
     compiled = torch.compile(layer, fullgraph=True)
     assert torch.equal(compiled(x[:1]), layer(x[:1]))
+
+
+@pytest.mark.parametrize("m", [1, 64])
+def test_shared_input_quantization(dev, m, monkeypatch):
+    """Layers marked `share_input_quantization` quantize a common input once; outputs equal the
+    per-layer forward bit for bit; a changed or different input is quantized again."""
+    from orbitquant_amd import OrbitLinear, OrbitQuantConfig, layers as layers_mod, ops
+
+    torch.manual_seed(11)
+    cfg = OrbitQuantConfig(weight_bits=4, activation_bits=4)
+    q, k, v = (OrbitLinear.from_linear(torch.nn.Linear(1024, n), config=cfg).to(dev) for n in (1024, 512, 256))
+    other = OrbitLinear.from_linear(torch.nn.Linear(2048, 256), config=cfg).to(dev)
+    x = torch.randn(m, 1024, device=dev, dtype=torch.bfloat16)
+    want = [layer(x) for layer in (q, k, v)]
+    calls = []
+    real = ops.rotate_quantize
+    monkeypatch.setattr(layers_mod.ops, "rotate_quantize", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    for layer in (q, k, v, other):
+        layer.share_input_quantization = True
+    layers_mod._last_quantization.clear()
+    got = [layer(x) for layer in (q, k, v)]
+    assert len(calls) == 1
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    other(torch.randn(m, 2048, device=dev, dtype=torch.bfloat16))   # another input in between: the entry is replaced
+    assert torch.equal(k(x), want[1]) and len(calls) == 3
+    x.add_(1)                                                        # same storage, new contents: the version counter moved
+    fresh = k(x)
+    assert len(calls) == 4 and not torch.equal(fresh, want[1])
+    k.share_input_quantization = False
+    assert torch.equal(k(x), fresh)
+    y = x.clone()                                                    # same values, another tensor
+    v(x)                                                             # still the entry k left
+    assert len(calls) == 4
+    v(y)
+    assert len(calls) == 5
