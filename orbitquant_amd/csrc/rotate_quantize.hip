@@ -133,7 +133,15 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              float *norms_out, const uint16_t *input_map, const void *plan, hipStream_t stream) {
   // With a rotate plan, launches of more than a few rows take the plan-based kernel (same results);
   // decode-sized launches and fused input maps stay with the kernel below, which is built for latency.
-  if (plan != nullptr && input_map == nullptr && M > 16) {
+  // The plan kernel gives every 512-slot unit (or block, if larger) of a row to one wavefront.  With many rows that is
+  // all the parallelism it needs; with at most sixteen rows it wins only when a row has several units (K = 14336
+  // in blocks of 2048, one token: 7.9 us against 10.1 us; K = 1152: 3.8 against 4.4) and loses when the row is one
+  // block (K = 4096 = one block: 9.9 against 5.6 us), which the kernel below spreads over a whole workgroup.
+  int64_t fast_min_m = 17;
+  if (const char *v = debug_env(ENV_RQ_FAST_MIN_M)) fast_min_m = atoi(v);
+  const int64_t unit = block > 512 ? block : 512;
+  const bool several_units = (K + unit - 1) / unit >= 3;
+  if (plan != nullptr && input_map == nullptr && (M >= fast_min_m || several_units)) {
     RqArgs checked;
     bool vec_checked = false;
     if (int rc = rotate_quantize_prepare(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,

@@ -217,6 +217,7 @@ static int launch_fast(FastArgs &a, int x_dtype, hipStream_t stream) {
   // eight for rows of sixteen units and more (measured: 5120 values in 5 units of 1024, 210 us on four
   // against 237 us on five; 13824 values in 27 units of 512, 608 us on eight against 655 us on four).
   int waves = a.units >= 16 ? 8 : (a.units < 4 ? a.units : 4);
+  if (a.M <= 16) waves = a.units < 8 ? a.units : 8;  // few rows: every unit its own wavefront
   if (const char *forced = debug_env(ENV_RQ_WAVES)) {
     const int w = atoi(forced);
     if (w >= 1 && w <= 8) waves = w < a.units ? w : a.units;
