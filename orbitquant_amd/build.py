@@ -36,6 +36,7 @@ SOURCES = {
     "packed_gemm.hip": [],
     "packed_gemm_bytes.hip": [],
     "packed_gemm_tiled.hip": [],
+    "packed_gemm_staged.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
     "token_linear.hip": [],

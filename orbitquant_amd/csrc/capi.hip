@@ -73,6 +73,9 @@ int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const
 int gemm_tiled_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
                         const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                         int out_dtype, hipStream_t stream);
+int gemm_staged_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
+                         const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
+                         int out_dtype, hipStream_t stream);
 int adaln_int4_dispatch(const uint16_t *x, const uint8_t *packed, const uint16_t *scales, const uint16_t *bias, int64_t M,
                         int64_t N, int64_t K, int64_t group, uint16_t *out, hipStream_t stream);
 int adaln_quantize_dispatch(const void *w, int w_dtype, int64_t N, int64_t K, int64_t group, uint8_t *packed, float *scales,
@@ -330,13 +333,18 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   hipStream_t s = as_stream(stream);
   if (x_dtype == OQ_BF16 && M >= 256 && K % 64 == 0 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) &&
       gemm_supported(K, bits)) {
-    // Large M: one pass puts the activations into the matrix core's operand order, then the tile kernel runs on them
-    // (not while the stream is being captured into a graph: the pass needs memory).
+    // Large M: the tile kernel of the code path on activation values.  Either one pass first puts the activations
+    // into the matrix core's operand order (fastest on large problems; needs a buffer, so not while the stream is
+    // being captured into a graph), or every wavefront stages its own rows through LDS (no buffer).
+    const char *force = debug_env(ENV_GEMM_TILE);
+    const bool force_staged = force != nullptr && force[0] != '\0' && force[1] == 's';
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
+    if (!force_staged && hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
       const int rc = gemm_tiled_dispatch(x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
       if (rc >= 0) return rc;
     }
+    if (M * K * 2 < (int64_t{1} << 32))
+      return gemm_staged_dispatch(x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
   }
   if (x_dtype != OQ_F32 && M > 8 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) && gemm_av_supported(K, bits))
   {

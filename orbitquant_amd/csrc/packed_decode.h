@@ -24,15 +24,21 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 typedef __attribute__((address_space(3))) const uint32_t lds_cu32;
+typedef uint32_t lds_u32x4 __attribute__((ext_vector_type(4)));
 
 #if defined(__HIP_DEVICE_COMPILE__)
 __device__ __forceinline__ uint32_t lds_read_u32(uint32_t byte_addr) { return *(lds_cu32 *)(byte_addr); }
+__device__ __forceinline__ uint4 lds_read_u128(uint32_t byte_addr) {  // 16-byte aligned
+  const lds_u32x4 v = *(__attribute__((address_space(3))) const lds_u32x4 *)(byte_addr);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
 
 __device__ __forceinline__ uint32_t lds_byte_address(const void *p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
 #else  // the host pass only needs the declarations to parse
 __device__ uint32_t lds_read_u32(uint32_t byte_addr);
+__device__ uint4 lds_read_u128(uint32_t byte_addr);
 __device__ uint32_t lds_byte_address(const void *p);
 #endif
 

@@ -46,7 +46,11 @@ namespace oq {
 // (r = lane % 32, g = lane / 32), the eight values k_step*64 + 32g + 8q .. +7 of row 32*row_tile + r
 // (tile_activations_kernel writes it).  Then a wavefront's activation load is 1 KB of consecutive
 // bytes, the operand needs no lookup, and only the weights go through the tables.
-enum AMode { A_NIBBLE = 0, A_U8 = 1, A_TILED = 2 };
+// A_STAGED: 16-bit values (bf16) as the caller has them, [M, K] row-major.  Every wavefront loads the 128-byte
+// K-step pieces of its own FM*32 rows line by line (eight rows per load instruction), parks them in a slab of
+// LDS that belongs to it alone (row pitch 144 bytes), and reads its operands back with one 16-byte LDS read per
+// row tile and MFMA: no workgroup-wide staging, no barrier in the loop, no copy of the activations in memory.
+enum AMode { A_NIBBLE = 0, A_U8 = 1, A_TILED = 2, A_STAGED = 3 };
 
 struct GemmArgs {
   const uint8_t *a;          // [M, K/2] nibble codes, [M, K] one code per byte, or the tiled 16-bit values
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // are written while the packed data is still in flight.
   const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
   uint32_t my_a;
-  if constexpr (AM == A_TILED) {
+  if constexpr (AM == A_TILED || AM == A_STAGED) {
     my_a = 0u;                     // no activation table
   } else if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
     const int c0 = tid & 15, c1 = tid >> 4;
@@ -123,16 +127,26 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   EpiFactors<FM> epi;
   gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
 
-  constexpr int kAStep = AM == A_NIBBLE ? 32 : AM == A_U8 ? 64 : 4096;  // bytes from one K-step of 64 to the next in a lane's activation stream
+  constexpr int kAStep = AM == A_NIBBLE ? 32 : AM == A_U8 ? 64 : AM == A_TILED ? 4096 : 128;  // bytes from one K-step of 64 to the next in a lane's activation stream
   constexpr int kAVec = AM == A_NIBBLE ? 1 : AM == A_U8 ? 2 : 4;        // 16-byte loads per lane per K-step
   constexpr int kAVecStride = AM == A_TILED ? 1024 : 16;
+  // A_STAGED: load v of row tile e is row 32 e + 8 v + lane / 8, 16-byte chunk lane % 8 of the row's 128-byte K-step piece
+  constexpr int kSlabPitch = 144, kSlabBytes = FM * 32 * kSlabPitch;
+  __shared__ __attribute__((aligned(16))) unsigned char aslab[AM == A_STAGED ? 4 * kSlabBytes : 16];
+  unsigned char *my_slab = aslab + (AM == A_STAGED ? wave * kSlabBytes : 0);
+  uint32_t a_off32[AM == A_STAGED ? FM : 1][4];  // byte offsets from g.a (the host checks M * K * 2 < 4 GB)
   const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K;
   const int64_t w_row_bytes = g.K * BITS / 8;
   const uint8_t *ap[FM];
   const uint8_t *wp[FN];
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
-    if constexpr (AM == A_TILED) ap[i] = g.a + min(m_base / 32 + i, (g.M + 31) / 32 - 1) * (g.K / 64) * kAStep + lane * 16;
+    if constexpr (AM == A_STAGED) {
+      ap[i] = g.a;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        a_off32[i][v] = static_cast<uint32_t>(min(m_base + 32 * i + 8 * v + (lane >> 3), g.M - 1) * (g.K * 2) + (lane & 7) * 16);
+    } else if constexpr (AM == A_TILED) ap[i] = g.a + min(m_base / 32 + i, (g.M + 31) / 32 - 1) * (g.K / 64) * kAStep + lane * 16;
     else ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
   }
 #pragma unroll
@@ -144,7 +158,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
   if constexpr (KSPLIT > 1) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * kAStep;
+    for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * kAStep;  // (A_STAGED: every ap[i] is the same base)
 #pragma unroll
     for (int j = 0; j < FN; ++j) wp[j] += static_cast<int64_t>(wave) * steps * (8 * BITS);
   }
@@ -154,7 +168,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     const int64_t s = min(ks, steps - 1);  // past the end: re-read the last step (never multiplied)
     if (e < FM) {
 #pragma unroll
-      for (int v = 0; v < kAVec; ++v) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + kAVecStride * v);
+      for (int v = 0; v < kAVec; ++v) {
+        if constexpr (AM == A_STAGED) pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + (a_off32[e][v] + static_cast<uint32_t>(s) * kAStep));
+        else pa[B][e][v] = *reinterpret_cast<const uint4 *>(ap[e] + s * kAStep + kAVecStride * v);
+      }
     }
     else load_w<BITS>(wp[e - FM] + s * (8 * BITS), pw[B][e - FM]);
   };
@@ -187,11 +204,28 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   //
   // One-code-per-byte activations take two lookups per operand dword (single-code table, the
   // value in both halves); the two are merged with one v_perm_b32 when the operand is used.
-  constexpr int kRA = AM == A_NIBBLE ? 4 : AM == A_U8 ? 8 : 0;  // LDS reads per activation tile and phase
+  constexpr int kRA = AM == A_NIBBLE ? 4 : AM == A_U8 ? 8 : AM == A_STAGED ? 1 : 0;  // LDS reads per activation tile and phase
   constexpr int kRAd = kRA > 0 ? kRA : 1;
   constexpr int kLookups = kRA * FM + 4 * FN, kGroups = FM * FN;  // group m takes lookups [m*L/G, (m+1)*L/G)
   constexpr int kLook = (kLookups + kGroups - 1) / kGroups;
-  uint32_t oa[2][FM][kRAd], ob[2][FN][4];  // two operand sets: one being multiplied, one being looked up
+  uint32_t oa[2][FM][kRAd], ob[2][FN][4];
+  uint4 oa4[2][AM == A_STAGED ? FM : 1];  // A_STAGED: the whole operand comes with one 16-byte read
+  const uint32_t slab_read = lds_byte_address(my_slab) + r * kSlabPitch + grp * 64;  // + 32 i * pitch + 16 q
+  // K-step buffer B (its loads have arrived) into the slab; the reads of the previous K-step were issued before
+  auto stash = [&](auto buf) {
+    constexpr int B = decltype(buf)::value;
+    if constexpr (AM == A_STAGED) {
+#pragma unroll
+      for (int e = 0; e < FM; ++e)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+        {  // (element-wise into a vector store: an aggregate copy from the register array would pin it in scratch)
+          const uint4 piece = pa[B][e][v];
+          *reinterpret_cast<lds_u32x4 *>(my_slab + (32 * e + 8 * v + (lane >> 3)) * kSlabPitch + (lane & 7) * 16) =
+              lds_u32x4{piece.x, piece.y, piece.z, piece.w};
+        }
+    }
+  };  // two operand sets: one being multiplied, one being looked up
 
   // dword d (0..7 for bytes, 0..3 for nibbles) of this lane's activation run in buffer B, tile i
   auto a_word = [&](auto buf, int i, int d) -> uint32_t {
@@ -209,7 +243,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
       if (is_a) {
         const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRAd;
         const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRAd;
-        if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
+        if constexpr (AM == A_STAGED) return slab_read + i * (32 * kSlabPitch) + q * 16;
+        else if constexpr (AM == A_NIBBLE) return row_address(a_word(buf, i, q), a_off, sub);
         else return row_address(a_word(buf, i, 2 * q + (sub >> 2)), a_off, sub & 3);  // byte 8q + sub of the run
       }
     }
@@ -223,7 +258,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     if (is_a) {
       const int i = t < kRA ? 0 : 1 + (t - kRA - 4 * FN) / kRAd;
       const int sub = t < kRA ? t : (t - kRA - 4 * FN) % kRAd;
-      oa[set][i][sub] = lds_read_u32(address);
+      if constexpr (AM == A_STAGED) oa4[set][i] = lds_read_u128(address);
+      else oa[set][i][sub] = lds_read_u32(address);
     } else {
       const int j = (t - kRA) >> 2, p = (t - kRA) & 3;
       if constexpr (BITS == 4) ob[set][j][p] = lds_read_u32(address);
@@ -234,6 +270,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   auto a_operand = [&](int set, int i) -> uint4 {
     if constexpr (AM == A_TILED) {
       return make_uint4(0u, 0u, 0u, 0u);  // (the operand comes straight from the load registers, see phase)
+    } else if constexpr (AM == A_STAGED) {
+      return oa4[set][i];
     } else if constexpr (AM == A_NIBBLE) {
       return make_uint4(oa[set][i][0], oa[set][i][1], oa[set][i][2], oa[set][i][3]);
     } else {
@@ -281,9 +319,11 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     if constexpr (FM + FN > FM * FN) fetch(prev, ks + NBUF - 1);
     phase(buf, 2, 0, prev, 0, false, buf, std::integral_constant<int, 1>{});
     phase(buf, 3, 1, prev, 0, false, buf, std::integral_constant<int, 2>{});
+    stash(next);  // every operand read of this K-step has been issued; the next K-step's pieces take the slab
     phase(next, 0, 0, prev, 0, false, buf, std::integral_constant<int, 3>{});
   };
 
+  stash(std::integral_constant<int, 0>{});
 #pragma unroll
   for (int t = 0; t < kLookups; ++t)
     lookup_read(std::integral_constant<int, 0>{}, 0, 0, t, lookup_address(std::integral_constant<int, 0>{}, 0, t));

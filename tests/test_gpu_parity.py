@@ -611,3 +611,37 @@ def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k):
                                      layer["r"].to(dev), torch.from_numpy(layer["cw"]).to(dev), code_format="nibble", activation_bits=4,
                                      weight_bits=bits, out_features=n, in_features=k, bias=bias.to(dev), output_dtype=torch.bfloat16)
         assert torch.equal(got, by_codes)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
+def test_matmul_packed_weight_large_m_bf16_under_graph_capture(dev, bits):
+    """While a stream is captured the large-M float-activation call may not allocate: every wavefront
+    stages its own activation rows through LDS instead.  Same tile kernel, same sums: the replayed
+    graph returns the bits of the eager call, replay after replay."""
+    from orbitquant_amd import ops
+
+    rng = np.random.default_rng(bits)
+    m, n, k = 520, 200, 1152
+    layer = make_layer(rng, n, k, bits, 4)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(F32)).to(torch.bfloat16).to(dev)
+    packed, r, cw = torch.from_numpy(layer["packed"]).to(dev), layer["r"].to(dev), torch.from_numpy(layer["cw"]).to(dev)
+    scale = torch.from_numpy(rng.uniform(0.5, 2.0, m).astype(F32)).to(dev)
+
+    def call():
+        return ops.matmul_packed_weight_values(x, packed, r, cw, bits=bits, out_features=n, in_features=k, token_scale=scale)
+    eager = call()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = call()
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert torch.equal(call(), eager)   # eager work between the replays
