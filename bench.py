@@ -35,6 +35,8 @@ def parse_args():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--m", type=int, default=0, help="token count override (c5: 1, 4 or 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-grouped-launch", action="store_true",
+                    help="c5: q, k and v share their input's quantization but each take a launch of their own")
     ap.add_argument("--no-shared-quantization", action="store_true",
                     help="c5: q, k and v each quantize their (common) input, as the reference's layers do")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
@@ -515,16 +517,29 @@ def bench_c5(args, device):
     gen = torch.Generator().manual_seed(5)
     m = args.m or 1
     mats = build_c5(device, gen)
-    # one input per role, as in a transformer block: q, k and v read the same tensor (and share its
-    # quantization, `share_input_quantization`), o, up and down each their own
-    x_attn, x_o, x_up = (torch.randn(m, 4096, generator=gen).to(torch.bfloat16).to(device) for _ in range(3))
-    x14336 = torch.randn(m, 14336, generator=gen).to(torch.bfloat16).to(device)
+    # one input per role and layer, as in a transformer: q, k and v of a layer read the same tensor
+    # (and share its quantization), o, up and down each their own; no tensor is read by two layers,
+    # so no quantization carries over from one layer to the next
+    def fresh(width):
+        return torch.randn(m, width, generator=gen).to(torch.bfloat16).to(device)
     roles = ("q", "k", "v", "o", "up", "down")
-    inputs = {"q": x_attn, "k": x_attn, "v": x_attn, "o": x_o, "up": x_up, "down": x14336}
-    layer_input = [inputs[roles[i % 6]] for i in range(len(mats))]
+    layer_input = []
+    for _ in range(len(mats) // 6):
+        x_attn = fresh(4096)
+        layer_input.extend([x_attn, x_attn, x_attn, fresh(4096), fresh(4096), fresh(14336)])
     if not args.no_shared_quantization:
         for i, l in enumerate(mats):
             l.share_input_quantization = roles[i % 6] in ("q", "k", "v")
+    # q, k and v of a block as one call (one quantization, one launch): OrbitLinearGroup
+    grouped = not (args.no_shared_quantization or args.no_grouped_launch)
+    if grouped:
+        from orbitquant_amd import OrbitLinearGroup
+        step_calls = []
+        for base in range(0, len(mats), 6):
+            step_calls.append((OrbitLinearGroup(*mats[base:base + 3]), layer_input[base]))
+            step_calls.extend((mats[base + j], layer_input[base + j]) for j in (3, 4, 5))
+    else:
+        step_calls = list(zip(mats, layer_input))
     packed_bytes = sum(l.packed_weight_indices.numel() + 2 * l.out_features for l in mats)
     pre = []
     for l, x in zip(mats, layer_input):
@@ -542,13 +557,13 @@ def bench_c5(args, device):
                               output_dtype=torch.bfloat16)
 
     def full_step():
-        for l, x in zip(mats, layer_input):
-            l(x)
+        for fn, x in step_calls:
+            fn(x)
 
     def full_step_out():
         last = None
-        for l, x in zip(mats, layer_input):
-            last = l(x)
+        for fn, x in step_calls:
+            last = fn(x)
         return last
 
     preroll(full_step)
@@ -586,7 +601,7 @@ def bench_c5(args, device):
                 raise RuntimeError(lib.oq_last_error().decode())
     abi_step()
     torch.cuda.synchronize()
-    assert torch.equal(keep[-1][2], mats[-1](x14336)) and torch.equal(keep[2][2], mats[2](x_attn)), "C-ABI stack differs from the module stack"
+    assert torch.equal(keep[-1][2], mats[-1](layer_input[-1])) and torch.equal(keep[2][2], mats[2](layer_input[2])), "C-ABI stack differs from the module stack"
     abi_dt = time_steps(abi_step, args.steps, args.warmup)
 
     # kernel-only: every matmul launch of the stack, events on the launch stream
@@ -609,6 +624,7 @@ def bench_c5(args, device):
         "data": "synthetic", "config": {"workload": f"c5 40-layer decode stack W2/W3/W4 A4, M={m}", "M": m,
                                         "packed_bytes_per_step": packed_bytes, "launch": launch,
                                         "shared_quantization": "none" if args.no_shared_quantization else "q, k, v of a block quantize their common input once",
+                                        "grouped_launch": "q, k, v of a block in one launch" if grouped else "none",
                                         "eager_ms_per_step": eager_dt * 1e3,
                                         "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
                                         "c_abi_ms_per_step": abi_dt * 1e3,

@@ -184,6 +184,25 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                      void *stream);
 
 /*
+ * `count` packed linears on the SAME activation codes (the q, k and v projections of an attention
+ * block, the gate and up projections of an MLP): out[i] = oq_packed_linear(codes, ..., packed_w[i],
+ * w_bits[i], row_norms[i], w_centroids[i], bias[i], M, N[i], K), bit for bit.  The argument arrays
+ * (count entries each, read during the call only) live in host memory and hold device pointers;
+ * `bias` may be NULL (no matrix has one) or hold NULL entries.  For at most sixteen tokens, nibble
+ * codes, 2-, 3- or 4-bit weights and two to four matrices the whole group is ONE launch of the
+ * streaming kernel (at decode sizes a launch is mostly fixed cost); any other group runs as
+ * `count` launches.  No counterpart in the reference, whose layers each call
+ * matmul_packed_* on their own (src/orbitquant/layers.py:1079-1455); it replaces `count`
+ * consecutive calls of oq_packed_linear.
+ */
+int oq_packed_linear_group(const void *codes, int code_format, const float *token_norms,
+                           const float *act_centroids, int a_bits, int count,
+                           const uint8_t *const *packed_w, const int *w_bits,
+                           const uint16_t *const *row_norms, const float *const *w_centroids,
+                           const void *const *bias, int bias_dtype, int64_t M, const int64_t *N,
+                           int64_t K, void *const *out, int out_dtype, void *stream);
+
+/*
  * oq_packed_linear followed by an elementwise function of the 16-bit outputs given as a
  * table (output_map[bits of y] = bits of f(y), 65536 entries of the output dtype, 16-byte
  * aligned, on the device): out = f(linear) bit for bit, f(...) applied before the store
@@ -233,6 +252,24 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
                         void *codes_scratch, float *norms_scratch,
                         void *out, int out_dtype, const uint16_t *output_map, void *stream);
+
+/*
+ * oq_quantized_linear for `count` linears that read the same input (q, k and v of an attention
+ * block; gate and up of an MLP): the input is quantized once into the caller's scratch buffers
+ * (required; sizes as for oq_quantized_linear), then oq_packed_linear_group.  out[i] equals what
+ * oq_quantized_linear gives for matrix i, bit for bit.  Arrays as in oq_packed_linear_group.
+ * No counterpart in the reference (see oq_packed_linear_group).
+ */
+int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_map,
+                              int64_t M, int64_t K,
+                              const int32_t *perm, const int8_t *signs, const float *boundaries,
+                              const float *act_centroids, int a_bits,
+                              int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan,
+                              int count, const uint8_t *const *packed_w, const int *w_bits,
+                              const uint16_t *const *row_norms, const float *const *w_centroids,
+                              const void *const *bias, int bias_dtype, const int64_t *N,
+                              void *codes_scratch, float *norms_scratch,
+                              void *const *out, int out_dtype, void *stream);
 
 /*
  * oq_quantized_linear for callers that cannot allocate device memory or bring a workspace:

@@ -39,6 +39,7 @@ SOURCES = {
     "packed_gemm_staged.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
+    "packed_gemv_group.hip": [],
     "token_linear.hip": [],
     "token_linear_w2.hip": [],
     "token_linear_w3.hip": [],

@@ -50,7 +50,7 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
 }
 
 const char *debug_env(int which) {
-  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES", "OQ_RQ_FAST_MIN_M"};
+  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES", "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R"};
   static const char *values[ENV_COUNT];
   static std::once_flag once;
   std::call_once(once, [] {
@@ -116,7 +116,10 @@ int gemv_dispatch(const void *codes, int code_format, const float *row_scale, co
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                   int out_dtype, hipStream_t stream);
-
+int gemv_group_dispatch(const void *codes, int code_format, const float *row_scale, const float *act_cents, int a_levels,
+                        int count, const uint8_t *const *w, const int *bits, const uint16_t *const *row_norms,
+                        const float *const *w_cents, const void *const *bias, int bias_dtype, int64_t M,
+                        const int64_t *N, int64_t K, void *const *out, int out_dtype, hipStream_t stream, bool *launched);
 // Scratch of oq_quantized_linear_static: the activation codes and token norms that pass from the
 // quantizer launch to the matmul launch.  One copy per GPU, at its own address there; host code
 // only ever uses the address hipGetSymbolAddress returns for the current device.
@@ -257,6 +260,36 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                             w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, nullptr, stream);
 }
 
+int oq_packed_linear_group(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
+                           int a_bits, int count, const uint8_t *const *packed_w, const int *w_bits,
+                           const uint16_t *const *row_norms, const float *const *w_centroids, const void *const *bias,
+                           int bias_dtype, int64_t M, const int64_t *N, int64_t K, void *const *out, int out_dtype,
+                           void *stream) {
+  if (count < 1 || count > 64) return fail(OQ_ERR_INVALID, "packed_linear_group: count=%d (1..64)", count);
+  if (packed_w == nullptr || w_bits == nullptr || row_norms == nullptr || w_centroids == nullptr || N == nullptr || out == nullptr)
+    return fail(OQ_ERR_INVALID, "packed_linear_group: null argument array");
+  for (int i = 0; i < count; ++i)
+    if (int rc = check_matmul_common("packed_linear_group", packed_w[i], w_bits[i], row_norms[i], w_centroids[i],
+                                     bias != nullptr ? bias[i] : nullptr, bias_dtype, M, N[i], K, out[i], out_dtype))
+      return rc;
+  if (M == 0) return OQ_OK;
+  if (codes == nullptr || act_centroids == nullptr) return fail(OQ_ERR_INVALID, "packed_linear_group: null codes/centroids");
+  if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "packed_linear_group: a_bits=%d", a_bits);
+  if (code_format != OQ_CODES_U8 && code_format != OQ_CODES_NIBBLE) return fail(OQ_ERR_INVALID, "packed_linear_group: code_format=%d", code_format);
+  bool launched = false;
+  if (int rc = gemv_group_dispatch(codes, code_format, token_norms, act_centroids, 1 << a_bits, count, packed_w, w_bits,
+                                   row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, as_stream(stream),
+                                   &launched))
+    return rc;
+  if (launched) return OQ_OK;
+  for (int i = 0; i < count; ++i)
+    if (int rc = packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w[i], w_bits[i],
+                                    row_norms[i], w_centroids[i], bias != nullptr ? bias[i] : nullptr, bias_dtype, M,
+                                    N[i], K, out[i], out_dtype, nullptr, stream))
+      return rc;
+  return OQ_OK;
+}
+
 int oq_packed_linear_mapped(const void *codes, int code_format, const float *token_norms,
                             const float *act_centroids, int a_bits, const uint8_t *packed_w, int w_bits,
                             const uint16_t *row_norms, const float *w_centroids, const void *bias, int bias_dtype,
@@ -298,6 +331,36 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
     return rc;
   return packed_linear_impl(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
                             w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
+}
+
+int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
+                              const int32_t *perm, const int8_t *signs, const float *boundaries,
+                              const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
+                              const void *rotate_plan, int count, const uint8_t *const *packed_w, const int *w_bits,
+                              const uint16_t *const *row_norms, const float *const *w_centroids, const void *const *bias,
+                              int bias_dtype, const int64_t *N, void *codes_scratch, float *norms_scratch,
+                              void *const *out, int out_dtype, void *stream) {
+  if (count < 1 || count > 64) return fail(OQ_ERR_INVALID, "quantized_linear_group: count=%d (1..64)", count);
+  if (packed_w == nullptr || w_bits == nullptr || row_norms == nullptr || w_centroids == nullptr || N == nullptr || out == nullptr)
+    return fail(OQ_ERR_INVALID, "quantized_linear_group: null argument array");
+  for (int i = 0; i < count; ++i)
+    if (int rc = check_matmul_common("quantized_linear_group", packed_w[i], w_bits[i], row_norms[i], w_centroids[i],
+                                     bias != nullptr ? bias[i] : nullptr, bias_dtype, M, N[i], K, out[i], out_dtype))
+      return rc;
+  if (M == 0) return OQ_OK;
+  if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "quantized_linear_group: a_bits=%d", a_bits);
+  if (act_centroids == nullptr) return fail(OQ_ERR_INVALID, "quantized_linear_group: null activation centroids");
+  const int levels = 1 << a_bits;
+  hipStream_t s = as_stream(stream);
+  if (codes_scratch == nullptr || norms_scratch == nullptr)
+    return fail(OQ_ERR_INVALID, "quantized_linear_group: null scratch buffers");
+  const int fmt = (a_bits <= 4 && (K & 1) == 0) ? OQ_CODES_NIBBLE : OQ_CODES_U8;
+  if (int rc = rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, nullptr, levels, block, eps,
+                                        inv_sqrt_block, codes_scratch, fmt, nullptr, OQ_VALUES_NONE, norms_scratch,
+                                        input_map, rotate_plan, s))
+    return rc;
+  return oq_packed_linear_group(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, count, packed_w, w_bits,
+                                row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, stream);
 }
 
 int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,

@@ -9,7 +9,8 @@ using namespace gemv;
 
 template <bool BYTES, int BITS, int R, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
-  packed_gemv_body<BYTES, BITS, R, WAVES, false>(g, [](auto) {});
+  OQ_GEMV_TABLE_BLOCK(lds);
+  packed_gemv_body<BYTES, BITS, R, WAVES, false>(g, lds, blockIdx.x, [](auto) {});
 }
 
 template <bool BYTES, int BITS, int R, int WAVES>

@@ -68,19 +68,25 @@ inline int gemv_waves(int64_t N, int64_t K) { return N <= 16 * 256 && K >= 2048 
 // once, at the point from which it no longer waits for loads of its own (a wavefront's loads
 // return in order: requested earlier, the weights would hold up everything `produce` reads).
 // The lookup tables are built before that, so their construction also overlaps it.
+// `lds` is the kernel's table block (OQ_GEMV_TABLE_BLOCK: declared by the kernel, not here, so
+// that a kernel holding several instances of this body has one block and not one per instance);
+// `group` numbers the workgroup's 16*R rows within the matrix (blockIdx.x in a launch of one
+// matrix).
+#define OQ_GEMV_TABLE_BLOCK(name) \
+  __shared__ __attribute__((aligned(65536))) uint32_t name[::oq::gemv::kGemvTableBytes / 4]
+
 template <bool BYTES, int BITS, int R, int WAVES, bool LATE, typename Produce>
-__device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, Produce produce) {
+__device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *lds, int64_t group, Produce produce) {
   constexpr int kAVec = BYTES ? 2 : 1;      // 16-byte loads of activation codes per lane and K-step
   constexpr int kAStep = 64 * kAVec;        // bytes of one activation row per K-step of 128
   static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
-  __shared__ __attribute__((aligned(65536))) uint32_t lds[kGemvTableBytes / 4];
   float *partial = reinterpret_cast<float *>(lds);  // [WAVES][R][64][4], after the main loop
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, grp = lane >> 4;
   const uint32_t lds_base = lds_byte_address(lds);  // a multiple of 65536 by the alignment
   const uint32_t w_off = lds_base + 4 * (lane & 31), a_off = lds_base + 128 + 4 * (lane & 31);
-  const int64_t n_base = static_cast<int64_t>(blockIdx.x) * (16 * R);
+  const int64_t n_base = group * (16 * R);
 
   const int steps = static_cast<int>(g.K / 128);
   const int s_begin = static_cast<int>(static_cast<int64_t>(steps) * wave / WAVES);

@@ -28,7 +28,8 @@ __global__ __launch_bounds__(64 * WAVES) void token_linear_kernel(rq::RqArgs q, 
   g.a = codes;
   g.row_scale = norm;
   const int tid = threadIdx.x;
-  gemv::packed_gemv_body<false, BITS, R, WAVES, true>(g, [&](auto issue_weights) {
+  OQ_GEMV_TABLE_BLOCK(tables);
+  gemv::packed_gemv_body<false, BITS, R, WAVES, true>(g, tables, blockIdx.x, [&](auto issue_weights) {
     rq::rotate_quantize_row<DT, true, LOG_G, true>(q, smem, 0, tid, 64 * WAVES, issue_weights);
   });
 }

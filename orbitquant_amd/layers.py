@@ -292,3 +292,59 @@ class OrbitLinear(nn.Module):
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
                 f"w{self.weight_bits}a{self.activation_bits}, block={self.rotation.block_size}")
+
+
+class OrbitLinearGroup:
+    """Linears that read the same input (q, k and v of an attention block; gate and up of an MLP),
+    called together: `q, k, v = OrbitLinearGroup(attn.q, attn.k, attn.v)(x)`.
+
+    The whole group is one native call (`oq_quantized_linear_group`): the input is quantized once,
+    and the packed linears of at most sixteen tokens are one launch.  Every output equals the module's
+    own `forward(x)` bit for bit.  The group holds references to the modules, not copies, and is not
+    itself a module: parameters and state dict stay where they are.  The members must share
+    `in_features`, rotation, activation width and fused input activation; under `torch.compile`, or
+    when a member has a fused output activation, the members are simply called one after the other.
+    The reference has no counterpart: its layers each quantize and multiply on their own
+    (src/orbitquant/layers.py:1079-1455)."""
+
+    def __init__(self, *linears: OrbitLinear) -> None:
+        if len(linears) < 1 or not all(isinstance(l, OrbitLinear) for l in linears):
+            raise TypeError("OrbitLinearGroup takes OrbitLinear modules")
+        first = linears[0]
+        for l in linears[1:]:
+            same = (l.in_features == first.in_features and l.rotation.seed == first.rotation.seed
+                    and l.rotation.block_size == first.rotation.block_size
+                    and l.activation_bits == first.activation_bits and l.activation_eps == first.activation_eps
+                    and l._input_activation == first._input_activation)
+            if not same:
+                raise ValueError("the linears of a group must share in_features, rotation, activation width, "
+                                 "eps and fused input activation")
+        self.linears = tuple(linears)
+
+    def __call__(self, x: torch.Tensor) -> tuple[torch.Tensor, ...]:
+        first = self.linears[0]
+        if torch.compiler.is_compiling() or any(l._output_activation_table is not None for l in self.linears):
+            return tuple(l(x) for l in self.linears)
+        if x.shape[-1] != first.in_features:
+            raise ValueError(f"expected last dimension {first.in_features}, got {x.shape[-1]}")
+        if x.device.type != "cuda":
+            raise RuntimeError(
+                "OrbitLinear runs on AMD GPUs only (torch device 'cuda'); there is no CPU fallback")
+        if x.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            raise ValueError("x must be float32, float16 or bfloat16")
+        table = first._input_activation_table
+        if table is not None and table.dtype != x.dtype:
+            raise ValueError(f"the fused input activation was built for {table.dtype}, got {x.dtype}")
+        weights = []
+        for l in self.linears:
+            l.last_effective_runtime_mode = "hip_packed"
+            bias = l.bias
+            if bias is not None and bias.dtype != x.dtype:
+                bias = bias.to(x.dtype)   # as the single layer's forward does
+            weights.append((l.packed_weight_indices, l.row_norms, l._weight_codebook_centroids, l.weight_bits,
+                            l.out_features, bias))
+        return tuple(ops.quantized_linear_group(
+            x, first._rotation_permutation, first._rotation_signs, first._activation_codebook_boundaries,
+            first._activation_codebook_centroids, weights, block_size=first.rotation.block_size,
+            eps=first.activation_eps, inv_sqrt_block=first.rotation.normalization,
+            activation_bits=first.activation_bits, input_map=table, plan=first._rotation_plan))

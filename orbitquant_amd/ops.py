@@ -284,6 +284,65 @@ def packed_linear(
     return out.reshape(*lead, out_features)
 
 
+def packed_linear_group(
+    codes: torch.Tensor,
+    token_norms: torch.Tensor,
+    activation_centroids: torch.Tensor,
+    weights,
+    *,
+    code_format: str,
+    activation_bits: int,
+    in_features: int,
+    output_dtype: torch.dtype = torch.bfloat16,
+) -> list[torch.Tensor]:
+    """`packed_linear` of the same activation codes on several matrices, through one native call
+    (one launch when the group is decode-sized, see oq_packed_linear_group).  `weights` is a sequence
+    of (packed_weight_indices, row_norms, weight_centroids, weight_bits, out_features, bias or None);
+    the biases present must share one dtype.  Returns the outputs in that order, each equal to what
+    `packed_linear` returns for its matrix."""
+    import ctypes
+
+    _require_gpu(codes, "codes")
+    fmt = {"u8": OQ_CODES_U8, "nibble": OQ_CODES_NIBBLE}[code_format]
+    width = in_features if fmt == OQ_CODES_U8 else in_features // 2
+    if codes.dtype != torch.uint8 or codes.shape[-1] != width:
+        raise ValueError(f"codes must be uint8 with last dimension {width}")
+    weights = list(weights)
+    if not 1 <= len(weights) <= 64:
+        raise ValueError("a group holds 1 to 64 matrices")
+    lead = codes.shape[:-1]
+    flat = codes.contiguous().reshape(-1, width)
+    m = flat.shape[0]
+    activation_centroids = _operand(activation_centroids, "activation_centroids", codes, dtype=torch.float32, numel=1 << activation_bits)
+    norms = _operand(token_norms.reshape(-1), "token_norms", codes, dtype=torch.float32, numel=m)
+    keep, outs, bias_dtype = [], [], None
+    for packed, row_norms, cents, bits, n, bias in weights:
+        expected = (n * in_features * bits + 7) // 8
+        packed = _operand(packed, "packed_weight_indices", codes, dtype=torch.uint8, min_numel=expected)
+        row_norms = _operand(row_norms, "row_norms", codes, dtype=torch.bfloat16, numel=n)
+        cents = _operand(cents, "weight_centroids", codes, dtype=torch.float32, numel=1 << bits)
+        bias = _operand(bias, "bias", codes, dtype=_FLOATS, numel=n)
+        if bias is not None:
+            if bias_dtype is not None and bias.dtype != bias_dtype:
+                raise ValueError("the biases of a group must share one dtype")
+            bias_dtype = bias.dtype
+        keep.append((packed, row_norms, cents, int(bits), int(n), bias))
+        outs.append(torch.empty((m, n), dtype=output_dtype, device=codes.device))
+    count = len(keep)
+    ptrs = ctypes.c_void_p * count
+    lib = _lib.load()
+    with _OnDevice(codes):
+        rc = lib.oq_packed_linear_group(
+            flat.data_ptr(), fmt, norms.data_ptr(), activation_centroids.data_ptr(), int(activation_bits), count,
+            ptrs(*[k[0].data_ptr() for k in keep]), (ctypes.c_int * count)(*[k[3] for k in keep]),
+            ptrs(*[k[1].data_ptr() for k in keep]), ptrs(*[k[2].data_ptr() for k in keep]),
+            ptrs(*[_ptr(k[5]) for k in keep]), _DTYPES[bias_dtype] if bias_dtype is not None else OQ_F32, m,
+            (ctypes.c_int64 * count)(*[k[4] for k in keep]), int(in_features),
+            ptrs(*[o.data_ptr() for o in outs]), _DTYPES[output_dtype], _stream(codes))
+    _lib.check(rc, "oq_packed_linear_group")
+    return [o.reshape(*lead, o.shape[-1]) for o in outs]
+
+
 def quantized_linear(
     x: torch.Tensor,
     permutation: torch.Tensor,
@@ -345,6 +404,75 @@ def quantized_linear(
             codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _ptr(output_map), _stream(x))
     _lib.check(rc, "oq_quantized_linear")
     return out.reshape(*x.shape[:-1], out_features)
+
+
+def quantized_linear_group(
+    x: torch.Tensor,
+    permutation: torch.Tensor,
+    signs: torch.Tensor,
+    boundaries: torch.Tensor,
+    act_centroids: torch.Tensor,
+    weights,
+    *,
+    block_size: int,
+    eps: float,
+    inv_sqrt_block: float,
+    activation_bits: int,
+    input_map: torch.Tensor | None = None,
+    plan: torch.Tensor | None = None,
+) -> list[torch.Tensor]:
+    """`quantized_linear` of one input on several matrices in one native call: one quantization,
+    then `packed_linear_group` (oq_quantized_linear_group).  `weights` as for
+    `packed_linear_group`.  Every output equals `quantized_linear` on its matrix."""
+    import ctypes
+
+    _require_gpu(x, "x")
+    dim = x.shape[-1]
+    rows = x.contiguous().reshape(-1, dim)
+    m = rows.shape[0]
+    weights = list(weights)
+    if not 1 <= len(weights) <= 64:
+        raise ValueError("a group holds 1 to 64 matrices")
+    permutation = _operand(permutation, "permutation", x, dtype=torch.int32, numel=dim)
+    signs = _operand(signs, "signs", x, dtype=torch.int8, numel=dim)
+    boundaries = _operand(boundaries, "boundaries", x, dtype=torch.float32, numel=(1 << activation_bits) - 1)
+    act_centroids = _operand(act_centroids, "act_centroids", x, dtype=torch.float32, numel=1 << activation_bits)
+    if input_map is not None:
+        if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device or x.dtype == torch.float32:
+            raise ValueError("input_map must hold 65536 entries of x's 16-bit dtype on x's device")
+        input_map = input_map.contiguous()
+    plan = _plan_operand(plan, x, dim)
+    keep, outs, bias_dtype = [], [], None
+    for packed, row_norms, cents, bits, n, bias in weights:
+        expected = (n * dim * bits + 7) // 8
+        packed = _operand(packed, "packed_weight_indices", x, dtype=torch.uint8, min_numel=expected)
+        row_norms = _operand(row_norms, "row_norms", x, dtype=torch.bfloat16, numel=n)
+        cents = _operand(cents, "weight_centroids", x, dtype=torch.float32, numel=1 << bits)
+        bias = _operand(bias, "bias", x, dtype=_FLOATS, numel=n)
+        if bias is not None:
+            if bias_dtype is not None and bias.dtype != bias_dtype:
+                raise ValueError("the biases of a group must share one dtype")
+            bias_dtype = bias.dtype
+        keep.append((packed, row_norms, cents, int(bits), int(n), bias))
+        outs.append(torch.empty((m, n), dtype=x.dtype, device=x.device))
+    nibble = activation_bits <= 4 and dim % 2 == 0
+    codes = torch.empty((m, dim // 2 if nibble else dim), dtype=torch.uint8, device=x.device)
+    norms = torch.empty(m, dtype=torch.float32, device=x.device)
+    count = len(keep)
+    ptrs = ctypes.c_void_p * count
+    lib = _lib.load()
+    with _OnDevice(x):
+        rc = lib.oq_quantized_linear_group(
+            rows.data_ptr(), _dt(rows), _ptr(input_map), m, dim, permutation.data_ptr(), signs.data_ptr(),
+            boundaries.data_ptr(), act_centroids.data_ptr(), int(activation_bits), int(block_size), float(eps),
+            float(inv_sqrt_block), _ptr(plan), count,
+            ptrs(*[k[0].data_ptr() for k in keep]), (ctypes.c_int * count)(*[k[3] for k in keep]),
+            ptrs(*[k[1].data_ptr() for k in keep]), ptrs(*[k[2].data_ptr() for k in keep]),
+            ptrs(*[_ptr(k[5]) for k in keep]), _DTYPES[bias_dtype] if bias_dtype is not None else OQ_F32,
+            (ctypes.c_int64 * count)(*[k[4] for k in keep]), codes.data_ptr(), norms.data_ptr(),
+            ptrs(*[o.data_ptr() for o in outs]), _dt(x), _stream(x))
+    _lib.check(rc, "oq_quantized_linear_group")
+    return [o.reshape(*x.shape[:-1], o.shape[-1]) for o in outs]
 
 
 def matmul_packed_weight_values(
