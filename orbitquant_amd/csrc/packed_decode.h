@@ -174,16 +174,41 @@ __device__ __forceinline__ float lane_table(const float *__restrict__ cents, int
 // four rows per 16-byte-per-lane store.  The caller puts a barrier between this and the first lookup.
 // A_SINGLE: the activation half holds single-code entries (one code per byte, up to 256 levels)
 // instead of the pair table of two 4-bit codes.
-template <int BITS, int WAVES, bool A_SINGLE = false>
+// W_ONLY: the activation half of every row is left alone (it then holds something else: the
+// small-M kernel parks decoded activation values there).
+template <int BITS, int WAVES, bool A_SINGLE = false, bool W_ONLY = false>
 __device__ __forceinline__ void build_row_tables(uint32_t *lds, const float *__restrict__ w_cents,
                                                  const float *__restrict__ act_cents, int a_levels) {
   constexpr int kLevels = 1 << BITS;
   constexpr bool kPair = BITS <= 4;
   constexpr int kRowsPerWave = 256 / WAVES;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const float a_tab = A_SINGLE ? lane_table<64>(act_cents, a_levels) : lane_table<16>(act_cents, a_levels);
+  float a_tab = 0.0f;
+  if constexpr (!W_ONLY) a_tab = A_SINGLE ? lane_table<64>(act_cents, a_levels) : lane_table<16>(act_cents, a_levels);
   float w_tab = 0.0f;
   if constexpr (kLevels <= 64) w_tab = lane_table<kLevels>(w_cents, kLevels);
+  if constexpr (W_ONLY) {
+    // only the rows an index can reach (16, 64 or 256), eight rows per 16-byte-per-lane store
+    // (a weight half is eight lanes wide), the groups of eight rows dealt round the wavefronts
+    constexpr int kRows = kPair ? (kLevels * kLevels < 256 ? kLevels * kLevels : 256) : kLevels;
+    constexpr int kGroups = (kRows + 7) / 8;
+#pragma unroll
+    for (int i = 0; i < (kGroups + WAVES - 1) / WAVES; ++i) {
+      const int grp8 = wave + WAVES * i;
+      if (grp8 >= kGroups) break;  // the same for the whole wavefront
+      const int e = 8 * grp8 + (lane >> 3);
+      uint32_t ew;
+      if constexpr (kLevels <= 64) {
+        if constexpr (kPair) ew = pack16(__shfl(w_tab, e & (kLevels - 1)), __shfl(w_tab, (e >> BITS) & (kLevels - 1)), false);
+        else ew = pack16(__shfl(w_tab, e & (kLevels - 1)), __shfl(w_tab, e & (kLevels - 1)), false);
+      } else {
+        const float v = w_cents[e];
+        ew = pack16(v, v, false);
+      }
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + e * 256 + (lane & 7) * 16) = make_uint4(ew, ew, ew, ew);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < kRowsPerWave / 4; ++i) {
     const int e = wave * kRowsPerWave + 4 * i + (lane >> 4);  // the row this lane writes to

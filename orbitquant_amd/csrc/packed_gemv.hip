@@ -7,10 +7,10 @@ namespace {
 
 using namespace gemv;
 
-template <bool BYTES, int BITS, int R, int WAVES>
+template <bool BYTES, int BITS, int R, int WAVES, bool ASTAGE = false>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_kernel(GemvArgs g) {
   OQ_GEMV_TABLE_BLOCK(lds);
-  packed_gemv_body<BYTES, BITS, R, WAVES, false>(g, lds, blockIdx.x, [](auto) {});
+  packed_gemv_body<BYTES, BITS, R, WAVES, false, ASTAGE>(g, lds, blockIdx.x, [](auto) {});
 }
 
 template <bool BYTES, int BITS, int R, int WAVES>
@@ -18,6 +18,11 @@ int launch(const GemvArgs &g, hipStream_t stream) {
   const int64_t groups = (g.N + 16 * R - 1) / (16 * R);
   if (groups > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemv: N too large");
   auto kern = packed_gemv_kernel<BYTES, BITS, R, WAVES>;
+  // few tokens of nibble codes: the variant that decodes the activation values once per workgroup
+  // (same sums)
+  if constexpr (!BYTES) {
+    if (gemv_stages_activations(g.M, g.K)) kern = packed_gemv_kernel<BYTES, BITS, R, WAVES, true>;
+  }
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(groups)), dim3(64 * WAVES), 0, stream, g);
   return check_launch("packed_gemv");
 }

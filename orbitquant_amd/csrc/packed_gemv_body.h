@@ -62,6 +62,13 @@ constexpr int kGemvTableBytes = kRowTableBytes;
 // The one-token kernel uses the same rule, so that both give the same sums.
 inline int gemv_waves(int64_t N, int64_t K) { return N <= 16 * 256 && K >= 2048 ? 16 : 8; }
 
+// Whether a launch on nibble codes decodes the activation values once per workgroup (ASTAGE
+// below): they must fit the activation half of the table block.  OQ_GEMV_NO_ASTAGE keeps the
+// lookups, for comparisons.
+inline bool gemv_stages_activations(int64_t M, int64_t K) {
+  return M * K <= 16384 && debug_env(ENV_GEMV_NO_ASTAGE) == nullptr;
+}
+
 // BYTES: activation codes come one per byte (widths above 4 bits) instead of two per byte.
 // LATE: the activation codes and their row scales do not exist yet when the kernel starts;
 // `produce(issue_weights)`, called by every thread, writes them and calls `issue_weights()`
@@ -75,8 +82,19 @@ inline int gemv_waves(int64_t N, int64_t K) { return N <= 16 * 256 && K >= 2048 
 #define OQ_GEMV_TABLE_BLOCK(name) \
   __shared__ __attribute__((aligned(65536))) uint32_t name[::oq::gemv::kGemvTableBytes / 4]
 
-template <bool BYTES, int BITS, int R, int WAVES, bool LATE, typename Produce>
+//
+// ASTAGE (nibble codes, M*K <= 16384): the activation VALUES are decoded once per workgroup and
+// parked in the activation half of the table block (row c, bytes 128..255 = values 64c..64c+63 of
+// the [M, K] activations as bf16), which an operand of eight consecutive values reads back with
+// ONE 16-byte LDS read (lanes of the same token row read the same address) in place of four
+// table lookups and their address arithmetic: a third of the kernel's LDS time at two row blocks
+// per wavefront.  The values are the table's (the same conversion of the same centroids), so
+// the sums do not change.
+constexpr int64_t kStageValues = 16384;  // 256 rows x 64 values
+
+template <bool BYTES, int BITS, int R, int WAVES, bool LATE, bool ASTAGE = false, typename Produce>
 __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *lds, int64_t group, Produce produce) {
+  static_assert(!ASTAGE || (!BYTES && !LATE), "staged activation values: nibble codes that exist at launch");
   constexpr int kAVec = BYTES ? 2 : 1;      // 16-byte loads of activation codes per lane and K-step
   constexpr int kAStep = 64 * kAVec;        // bytes of one activation row per K-step of 128
   static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
@@ -107,6 +125,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
     uint32_t w[kDepth][R][BITS];
   };
   auto fetch_a = [&](int s0, Batch &bt) {
+    if constexpr (ASTAGE) return;
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       const int s = max(min(s0 + d, s_end - 1), 0);  // clamped: stays inside the row, result unused
@@ -128,6 +147,21 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
     fetch_w(s0, bt);
   };
 
+  // ASTAGE: the codes this thread decodes (groups of eight values, 4 bytes; requested before
+  // everything else so that they are not queued behind the stream), and the address of the lane's
+  // operand of K-step 0, MFMA 0: value (row, 32*grp) of the staged activations.
+  constexpr int kStageIters = ASTAGE ? static_cast<int>(kStageValues / 8) / (64 * WAVES) : 1;
+  uint32_t stage_codes[kStageIters];
+  const int stage_groups = ASTAGE ? g.M * static_cast<int>(g.K / 8) : 0;
+  uint32_t a_stage = 0;
+  if constexpr (ASTAGE) {
+#pragma unroll
+    for (int i = 0; i < kStageIters; ++i)
+      stage_codes[i] = reinterpret_cast<const uint32_t *>(g.a)[min(tid + i * 64 * WAVES, stage_groups - 1)];
+    const uint32_t v0 = static_cast<uint32_t>(min(r, g.M - 1)) * static_cast<uint32_t>(g.K) + 32u * grp;
+    a_stage = lds_base + 128u + ((v0 >> 6) << 8) + ((v0 & 63u) << 1);
+  }
+
   f32x4 acc[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -138,7 +172,9 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           uint4 af;
-          if constexpr (!BYTES) {
+          if constexpr (ASTAGE) {
+            af = lds_read_u128(a_stage + static_cast<uint32_t>(s0 + d) * 512u + q * 16);
+          } else if constexpr (!BYTES) {
             const uint4 v = bt.a[d][0];
             af = decode_bytes(q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w, a_off);
           } else {  // eight single-code lookups (value in both halves), merged two by two
@@ -198,7 +234,26 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   }
 
   // ---- tables (built while the stream is in flight) ---------------------------------------
-  build_row_tables<BITS, WAVES, BYTES>(lds, g.w_cents, g.act_cents, g.a_levels);
+  build_row_tables<BITS, WAVES, BYTES, ASTAGE>(lds, g.w_cents, g.act_cents, g.a_levels);
+  if constexpr (ASTAGE) {
+    const float a_tab = lane_table<16>(g.act_cents, g.a_levels);
+#pragma unroll
+    for (int i = 0; i < kStageIters; ++i) {
+      if (i * 64 * WAVES >= stage_groups) break;  // the same for every thread
+      const int j = tid + i * 64 * WAVES;
+      uint32_t d[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {  // every lane shuffles (a lane past the end decodes a clamped word and drops it)
+        const uint32_t byte = (stage_codes[i] >> (8 * b)) & 0xffu;
+        d[b] = pack16(__shfl(a_tab, static_cast<int>(byte & 15u)), __shfl(a_tab, static_cast<int>(byte >> 4)), false);
+      }
+      if (j < stage_groups) {
+        const uint32_t v = 8u * static_cast<uint32_t>(j);
+        *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + 128u + ((v >> 6) << 8) + ((v & 63u) << 1)) =
+            make_uint4(d[0], d[1], d[2], d[3]);
+      }
+    }
+  }
   if constexpr (LATE) {
     produce(issue_weights);
     __syncthreads();

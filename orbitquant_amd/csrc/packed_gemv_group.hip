@@ -15,23 +15,24 @@ namespace {
 
 using namespace gemv;
 
-template <int R, int WAVES>
+template <int R, int WAVES, bool ASTAGE>
 __global__ __launch_bounds__(64 * WAVES) void packed_gemv_group_kernel(GroupArgs ga) {
   OQ_GEMV_TABLE_BLOCK(lds);
   GemvArgs g;
   int bits, first;
   group_member(ga, blockIdx.x, g, bits, first);
   const int64_t group = static_cast<int>(blockIdx.x) - first;
-  if (bits == 2) packed_gemv_body<false, 2, R, WAVES, false>(g, lds, group, [](auto) {});
-  else if (bits == 3) packed_gemv_body<false, 3, R, WAVES, false>(g, lds, group, [](auto) {});
-  else packed_gemv_body<false, 4, R, WAVES, false>(g, lds, group, [](auto) {});
+  if (bits == 2) packed_gemv_body<false, 2, R, WAVES, false, ASTAGE>(g, lds, group, [](auto) {});
+  else if (bits == 3) packed_gemv_body<false, 3, R, WAVES, false, ASTAGE>(g, lds, group, [](auto) {});
+  else packed_gemv_body<false, 4, R, WAVES, false, ASTAGE>(g, lds, group, [](auto) {});
 }
 
 template <int R, int WAVES>
 int launch_group(GroupArgs &ga, hipStream_t stream) {
   const int64_t total = group_grid(ga, R);
   if (total < 0) return fail(OQ_ERR_UNSUPPORTED, "packed_linear_group: too many rows");
-  auto kern = packed_gemv_group_kernel<R, WAVES>;
+  auto kern = packed_gemv_group_kernel<R, WAVES, false>;
+  if (gemv_stages_activations(ga.m[0].M, ga.m[0].K)) kern = packed_gemv_group_kernel<R, WAVES, true>;
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(64 * WAVES), 0, stream, ga);
   return check_launch("packed_linear_group");
 }

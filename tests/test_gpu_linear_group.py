@@ -119,6 +119,31 @@ def test_group_result_does_not_depend_on_rows_per_workgroup(dev, rows_per_step):
     assert done.returncode == 0 and "same" in done.stdout, done.stderr[-2000:]
 
 
+@pytest.mark.parametrize("k,n,wbits", [(4096, 4096, 4), (4096, 14336, 3), (2048, 520, 2), (14336, 4096, 4), (1024, 96, 6),
+                                        (512, 40, 8), (16384, 64, 4)])
+def test_few_token_launch_equals_rows_of_a_batch(dev, k, n, wbits):
+    """Launches of few tokens (M*K <= 16384) read their activation operands from values decoded once
+    per workgroup; larger launches look every operand up in the table.  Token rows are independent, so
+    a row computed alone, in a staged launch of few rows and in a sixteen-row batch must agree bit for bit."""
+    from orbitquant_amd import ops
+
+    c = make_group(dev, 16, k, [(n, wbits, True)], 4, torch.bfloat16, seed=900 + wbits)
+    w = c["weights"][0]
+
+    def run(rows):
+        return ops.packed_linear(c["codes"][rows], c["norms"][rows], c["cents"], w[0], w[1], w[2], code_format="nibble",
+                                 activation_bits=4, weight_bits=wbits, out_features=n, in_features=k, bias=w[5],
+                                 output_dtype=torch.bfloat16)
+
+    batch = run(slice(0, 16))
+    few = max(1, min(16, 16384 // k))
+    for start in (0, 16 - few):
+        assert torch.equal(run(slice(start, start + few)), batch[start:start + few]), (start, few)
+    assert torch.equal(run(slice(5, 6)), batch[5:6])
+    if few >= 3:
+        assert torch.equal(run(slice(2, 5)), batch[2:5])
+
+
 WHOLE = [
     # one token, wide rows: quantizer launch, then the whole group in one launch
     dict(m=1, k=4096, shapes=[(4096, 2, False), (1024, 2, True), (1000, 3, False)], dtype=torch.bfloat16, block="paper"),
