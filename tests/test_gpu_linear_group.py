@@ -84,12 +84,11 @@ GROUPS = [
 ]
 
 
-@pytest.mark.parametrize("case", range(len(GROUPS)))
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+# every case in bf16, a third of them also with fp32 outputs and biases
+@pytest.mark.parametrize("case,dtype", [(c, torch.bfloat16) for c in range(len(GROUPS))] +
+                         [(c, torch.float32) for c in range(0, len(GROUPS), 3)])
 def test_group_equals_one_call_per_matrix(dev, case, dtype):
     spec = GROUPS[case]
-    if dtype == torch.float32 and case % 3:   # a third of the cases also with fp32 outputs and biases
-        pytest.skip("bf16 only")
     c = make_group(dev, spec["m"], spec["k"], spec["shapes"], spec["abits"], dtype, seed=100 + case)
     want = one_by_one(c)
     got = grouped(c)
@@ -160,8 +159,9 @@ WHOLE = [
 ]
 
 
-@pytest.mark.parametrize("case", range(len(WHOLE)))
-@pytest.mark.parametrize("mapped", [False, True])
+# every case plain; every other 16-bit case also through an input map
+@pytest.mark.parametrize("case,mapped", [(c, False) for c in range(len(WHOLE))] +
+                         [(c, True) for c in range(0, len(WHOLE), 2) if WHOLE[c]["dtype"] != torch.float32])
 def test_whole_forward_group_equals_one_call_per_matrix(dev, case, mapped):
     """ops.quantized_linear_group (oq_quantized_linear_group) against ops.quantized_linear per matrix,
     which is pinned to quantize + packed linear in test_gpu_token_linear.py."""
@@ -171,8 +171,6 @@ def test_whole_forward_group_equals_one_call_per_matrix(dev, case, mapped):
 
     spec = WHOLE[case]
     m, k, dtype = spec["m"], spec["k"], spec["dtype"]
-    if mapped and (dtype == torch.float32 or case % 2):
-        pytest.skip("input maps: 16-bit inputs, every other case")
     rot, acb = get_rpbh_rotation(k, 0, spec["block"]), get_codebook(k, 4)
     g = torch.Generator().manual_seed(500 + case)
     x = torch.randn(m, k, generator=g)
