@@ -273,12 +273,13 @@ def gemm_only_closure(layer, x, with_output_map=True):
             inv_sqrt_block=layer.rotation.normalization, code_format=fmt,
             input_map=layer._input_activation_table, plan=layer._rotation_plan)
         bias = layer.bias
+        packed, weight_bits, weight_centroids = layer._matmul_weight(x.numel() // k)  # what the layer's forward reads
 
         def fn():
             return ops.packed_linear(
-                codes, norms, layer._activation_codebook_centroids, layer.packed_weight_indices, layer.row_norms,
-                layer._weight_codebook_centroids, code_format=fmt, activation_bits=layer.activation_bits,
-                weight_bits=layer.weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
+                codes, norms, layer._activation_codebook_centroids, packed, layer.row_norms,
+                weight_centroids, code_format=fmt, activation_bits=layer.activation_bits,
+                weight_bits=weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
                 output_dtype=x.dtype, output_map=layer._output_activation_table if with_output_map else None)
         return fn
     _, unit, norms = ops.rotate_quantize(

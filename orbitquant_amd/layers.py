@@ -139,6 +139,47 @@ class OrbitLinear(nn.Module):
         # share its quantization: set this on each of them and the codes the first one computes serve the
         # others (see _shared_codes).  Off by default: the reference quantizes per layer.
         self.share_input_quantization = False
+        # 2- and 3-bit weights, many tokens: the tile kernel reads a copy of the indices repacked at four
+        # bits each (see _matmul_weight).  The copy is made on first need and costs out*in/2 bytes.
+        self.nibble_copy_for_many_tokens = True
+        self.register_buffer("_nibble_weight_copy", None, persistent=False)
+        self.register_buffer("_nibble_weight_centroids", None, persistent=False)
+
+    MANY_TOKENS = 256
+
+    def prepare_many_token_weights(self) -> None:
+        """Build the four-bit copy of a 2- or 3-bit index stream now (it is otherwise built by the first
+        forward of at least `MANY_TOKENS` rows; a forward that `torch.compile` is tracing cannot build
+        it and runs on the stored stream)."""
+        if self.weight_bits not in (2, 3) or self.packed_weight_indices.device.type != "cuda":
+            return
+        with torch.no_grad():
+            count = self.out_features * self.in_features
+            indices = ops.unpack_lowbit(self.packed_weight_indices.detach(), self.weight_bits, count)
+            self._nibble_weight_copy = ops.pack_lowbit(indices, 4)
+            cents = torch.zeros(16, dtype=torch.float32, device=indices.device)
+            cents[: 1 << self.weight_bits] = self._weight_codebook_centroids
+            self._nibble_weight_centroids = cents
+
+    def _matmul_weight(self, tokens: int):
+        """(packed indices, bits per index, centroids) the matmul of `tokens` rows reads.  The stored
+        stream, except for 2- and 3-bit weights at `MANY_TOKENS` rows or more: the tile kernel is bound
+        by instruction issue there, not by weight bytes, and extracting 3-bit fields that straddle bytes
+        (or four 2-bit fields per byte) costs it 11-22 % against whole nibbles, so it is given the same
+        indices at four bits each, with the codebook padded to sixteen entries.  Same operand values,
+        same sums.  Decode-sized calls, which are bound by the bytes, keep reading the stored stream."""
+        if (self.weight_bits in (2, 3) and self.nibble_copy_for_many_tokens and tokens >= self.MANY_TOKENS
+                and self.packed_weight_indices.device.type == "cuda"):
+            if self._nibble_weight_copy is None and not torch.compiler.is_compiling():
+                self.prepare_many_token_weights()
+            if self._nibble_weight_copy is not None:
+                return self._nibble_weight_copy, 4, self._nibble_weight_centroids
+        return self.packed_weight_indices, self.weight_bits, self._weight_codebook_centroids
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._nibble_weight_copy = None   # follows packed_weight_indices
+        self._nibble_weight_centroids = None
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def fuse_input_activation(self, fn, *, dtype: torch.dtype = torch.bfloat16) -> "OrbitLinear":
         """Make forward(x) return what forward(fn(x)) returns, bit for bit, without a separate
@@ -230,6 +271,8 @@ class OrbitLinear(nn.Module):
         for name, tensor in self._constants().items():
             setattr(self, name, tensor.to(device))
         self._build_rotation_plan()
+        self._nibble_weight_copy = None   # rebuilt on the new device / from uncast centroids when next needed
+        self._nibble_weight_centroids = None
         if self._input_activation is not None and device.type == "cuda":
             # a dtype cast must not touch the table's bits: fill it again
             self._input_activation_table = ops.activation_table(*self._input_activation, device)
@@ -254,11 +297,12 @@ class OrbitLinear(nn.Module):
         self.last_effective_runtime_mode = "hip_packed"
         if self.share_input_quantization and not torch.compiler.is_compiling():
             return self._forward_shared(x, table, out_table)
+        packed, weight_bits, weight_centroids = self._matmul_weight(x.numel() // self.in_features)
         return torch.ops.orbitquant_amd.quantized_linear(
             x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_centroids,
-            self._activation_codebook_boundaries, self.packed_weight_indices, self.row_norms,
-            self._weight_codebook_centroids, self.bias, self.rotation.block_size,
-            self.activation_eps, self.rotation.normalization, self.activation_bits, self.weight_bits,
+            self._activation_codebook_boundaries, packed, self.row_norms,
+            weight_centroids, self.bias, self.rotation.block_size,
+            self.activation_eps, self.rotation.normalization, self.activation_bits, weight_bits,
             self.out_features, table, out_table, self._rotation_plan)
 
     def _forward_shared(self, x, table, out_table):
@@ -284,9 +328,10 @@ class OrbitLinear(nn.Module):
         bias = self.bias
         if bias is not None and bias.dtype != x.dtype:
             bias = bias.to(x.dtype)   # as the fused op (and the reference on accelerators) does
-        return ops.packed_linear(codes, norms, self._activation_codebook_centroids, self.packed_weight_indices, self.row_norms,
-                                 self._weight_codebook_centroids, code_format=fmt, activation_bits=self.activation_bits,
-                                 weight_bits=self.weight_bits, out_features=self.out_features, in_features=self.in_features,
+        packed, weight_bits, weight_centroids = self._matmul_weight(x.numel() // self.in_features)
+        return ops.packed_linear(codes, norms, self._activation_codebook_centroids, packed, self.row_norms,
+                                 weight_centroids, code_format=fmt, activation_bits=self.activation_bits,
+                                 weight_bits=weight_bits, out_features=self.out_features, in_features=self.in_features,
                                  bias=bias, output_dtype=x.dtype, output_map=out_table)
 
     def extra_repr(self) -> str:
@@ -341,8 +386,8 @@ class OrbitLinearGroup:
             bias = l.bias
             if bias is not None and bias.dtype != x.dtype:
                 bias = bias.to(x.dtype)   # as the single layer's forward does
-            weights.append((l.packed_weight_indices, l.row_norms, l._weight_codebook_centroids, l.weight_bits,
-                            l.out_features, bias))
+            packed, weight_bits, weight_centroids = l._matmul_weight(x.numel() // first.in_features)
+            weights.append((packed, l.row_norms, weight_centroids, weight_bits, l.out_features, bias))
         return tuple(ops.quantized_linear_group(
             x, first._rotation_permutation, first._rotation_signs, first._activation_codebook_boundaries,
             first._activation_codebook_centroids, weights, block_size=first.rotation.block_size,
