@@ -162,8 +162,10 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
  *
  * Replaces matmul_packed_w4a4_int8 (torch_binding.cpp:39-46; packed_matmul.cu:744-1009)
  * for every weight width, with exact (bf16-rounded) centroids instead of the
- * int8 surrogate.  M <= 16 takes the streaming small-M kernel, larger M the MFMA
- * tile kernel.
+ * int8 surrogate.  M <= 64 takes the streaming small-M kernel (the weights are read and
+ * decoded once, sixteen token rows per matrix instruction, up to four blocks of sixteen per
+ * workgroup), larger M the MFMA tile kernel.  A token row's result does not depend on the
+ * rows computed with it as long as the call stays within 64 rows.
  *
  * codes        activation codes in code_format (see oq_rotate_quantize)
  * token_norms  fp32 [M]

@@ -40,6 +40,7 @@ SOURCES = {
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
     "packed_gemv_group.hip": [],
+    "packed_gemv_rows.hip": [],
     "token_linear.hip": [],
     "token_linear_w2.hip": [],
     "token_linear_w3.hip": [],

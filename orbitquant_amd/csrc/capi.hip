@@ -50,7 +50,7 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
 }
 
 const char *debug_env(int which) {
-  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES", "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE"};
+  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES", "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE", "OQ_GEMV_MAX_M"};
   static const char *values[ENV_COUNT];
   static std::once_flag once;
   std::call_once(once, [] {

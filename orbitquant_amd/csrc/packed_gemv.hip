@@ -1,5 +1,6 @@
-// Small-M (decode-sized, M <= 16) packed-weight linear on activation codes: kernel, launch
-// configuration and argument checks.  The arithmetic is in packed_gemv_body.h.
+// Small-M (decode-sized, M <= 16; up to 64 through packed_gemv_rows.hip) packed-weight linear on
+// activation codes: kernel, launch configuration and argument checks.  The arithmetic is in
+// packed_gemv_body.h.
 #include "packed_gemv_body.h"
 
 namespace oq {
@@ -59,9 +60,11 @@ int launch_bits(const GemvArgs &g, hipStream_t stream) {
 
 }  // namespace
 
+int gemv_rows_dispatch(const gemv::GemvArgs &g, int bits, bool bytes, hipStream_t stream);  // packed_gemv_rows.hip
+
 bool gemv_supported(int64_t M, int64_t K, int bits, int code_format, int a_levels) {
   const bool codes_ok = code_format == OQ_CODES_NIBBLE ? a_levels <= 16 : a_levels <= 256;
-  return M >= 1 && M <= 16 && K % 128 == 0 && codes_ok && (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
+  return M >= 1 && M <= gemv_max_tokens() && K % 128 == 0 && codes_ok && (bits == 2 || bits == 3 || bits == 4 || bits == 6 || bits == 8);
 }
 
 int gemv_dispatch(const void *codes, int code_format, const float *row_scale, const float *act_cents, int a_levels,
@@ -72,6 +75,7 @@ int gemv_dispatch(const void *codes, int code_format, const float *row_scale, co
   g.a = static_cast<const uint8_t *>(codes); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = static_cast<int>(M); g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
+  if (M > 16) return gemv_rows_dispatch(g, bits, code_format != OQ_CODES_NIBBLE, stream);
 #define OQ_GEMV_BITS(BYTES)                                                   \
   switch (bits) {                                                             \
     case 2: return launch_bits<BYTES, 2>(g, stream);                          \

@@ -62,6 +62,16 @@ constexpr int kGemvTableBytes = kRowTableBytes;
 // The one-token kernel uses the same rule, so that both give the same sums.
 inline int gemv_waves(int64_t N, int64_t K) { return N <= 16 * 256 && K >= 2048 ? 16 : 8; }
 
+// Tokens up to which the streaming kernel is taken (beyond: the tile kernel).  OQ_GEMV_MAX_M
+// (16, 32 or 64) overrides, for comparisons.
+inline int gemv_max_tokens() {
+  if (const char *v = debug_env(ENV_GEMV_MAX_M)) {
+    const int m = atoi(v);
+    if (m == 16 || m == 32 || m == 64) return m;
+  }
+  return 64;
+}
+
 // Whether a launch on nibble codes decodes the activation values once per workgroup (ASTAGE
 // below): they must fit the activation half of the table block.  OQ_GEMV_NO_ASTAGE keeps the
 // lookups, for comparisons.
@@ -92,13 +102,21 @@ inline bool gemv_stages_activations(int64_t M, int64_t K) {
 // the sums do not change.
 constexpr int64_t kStageValues = 16384;  // 256 rows x 64 values
 
-template <bool BYTES, int BITS, int R, int WAVES, bool LATE, bool ASTAGE = false, typename Produce>
+//
+// MB: blocks of sixteen token rows (M <= 16*MB).  Every decoded weight operand feeds MB matrix
+// instructions, one per block, each with its own activation operand and accumulators; a token
+// row's sums are the same whatever MB is.  Launches of 17 to 64 tokens stream the weights once
+// this way instead of taking the tile kernel, whose 128-row tiles are mostly padding there and
+// whose grid is too small for short-and-long matrices.
+template <bool BYTES, int BITS, int R, int WAVES, bool LATE, bool ASTAGE = false, int MB = 1, typename Produce>
 __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *lds, int64_t group, Produce produce) {
   static_assert(!ASTAGE || (!BYTES && !LATE), "staged activation values: nibble codes that exist at launch");
+  static_assert(MB == 1 || (!ASTAGE && !LATE), "several row blocks: plain launches with table lookups");
+  static_assert(R * MB <= WAVES, "every epilogue item (64 per row block and row step) needs a thread");
   constexpr int kAVec = BYTES ? 2 : 1;      // 16-byte loads of activation codes per lane and K-step
   constexpr int kAStep = 64 * kAVec;        // bytes of one activation row per K-step of 128
-  static_assert(WAVES * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
-  float *partial = reinterpret_cast<float *>(lds);  // [WAVES][R][64][4], after the main loop
+  static_assert(WAVES * MB * R * 64 * 16 <= kGemvTableBytes, "partial sums reuse the table block");
+  float *partial = reinterpret_cast<float *>(lds);  // [WAVES][MB][R][64][4], after the main loop
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, grp = lane >> 4;
@@ -111,7 +129,10 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   const int s_end = static_cast<int>(static_cast<int64_t>(steps) * (wave + 1) / WAVES);
 
   const int64_t w_row_bytes = g.K * BITS / 8;
-  const uint8_t *ap = g.a + static_cast<int64_t>(min(r, g.M - 1)) * (BYTES ? g.K : g.K / 2) + grp * (16 * kAVec);
+  const uint8_t *ap[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+    ap[mb] = g.a + static_cast<int64_t>(min(16 * mb + r, g.M - 1)) * (BYTES ? g.K : g.K / 2) + grp * (16 * kAVec);
   const uint8_t *wp[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) {
@@ -121,7 +142,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
 
   // a batch = kDepth K-steps: every load of the batch is issued before anything waits on it
   struct Batch {
-    uint4 a[kDepth][kAVec];
+    uint4 a[kDepth][MB][kAVec];
     uint32_t w[kDepth][R][BITS];
   };
   auto fetch_a = [&](int s0, Batch &bt) {
@@ -130,8 +151,10 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
     for (int d = 0; d < kDepth; ++d) {
       const int s = max(min(s0 + d, s_end - 1), 0);  // clamped: stays inside the row, result unused
 #pragma unroll
-      for (int v = 0; v < kAVec; ++v)
-        bt.a[d][v] = *reinterpret_cast<const uint4 *>(ap + static_cast<int64_t>(s) * kAStep + 16 * v);
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int v = 0; v < kAVec; ++v)
+          bt.a[d][mb][v] = *reinterpret_cast<const uint4 *>(ap[mb] + static_cast<int64_t>(s) * kAStep + 16 * v);
     }
   };
   auto fetch_w = [&](int s0, Batch &bt) {
@@ -162,48 +185,56 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
     a_stage = lds_base + 128u + ((v0 >> 6) << 8) + ((v0 & 63u) << 1);
   }
 
-  f32x4 acc[R];
+  f32x4 acc[MB][R];
 #pragma unroll
-  for (int j = 0; j < R; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < R; ++j) acc[mb][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   auto consume = [&](int s0, const Batch &bt, auto guarded) {
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
       if (!decltype(guarded)::value || s0 + d < s_end) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          uint4 af;
-          if constexpr (ASTAGE) {
-            af = lds_read_u128(a_stage + static_cast<uint32_t>(s0 + d) * 512u + q * 16);
-          } else if constexpr (!BYTES) {
-            const uint4 v = bt.a[d][0];
-            af = decode_bytes(q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w, a_off);
-          } else {  // eight single-code lookups (value in both halves), merged two by two
-            const uint4 v = bt.a[d][q >> 1];
-            const uint4 e0 = decode_bytes((q & 1) ? v.z : v.x, a_off), e1 = decode_bytes((q & 1) ? v.w : v.y, a_off);
-            af = make_uint4(__builtin_amdgcn_perm(e0.y, e0.x, 0x07060100u), __builtin_amdgcn_perm(e0.w, e0.z, 0x07060100u),
-                            __builtin_amdgcn_perm(e1.y, e1.x, 0x07060100u), __builtin_amdgcn_perm(e1.w, e1.z, 0x07060100u));
+          uint4 af[MB];
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            if constexpr (ASTAGE) {
+              af[mb] = lds_read_u128(a_stage + static_cast<uint32_t>(s0 + d) * 512u + q * 16);
+            } else if constexpr (!BYTES) {
+              const uint4 v = bt.a[d][mb][0];
+              af[mb] = decode_bytes(q == 0 ? v.x : q == 1 ? v.y : q == 2 ? v.z : v.w, a_off);
+            } else {  // eight single-code lookups (value in both halves), merged two by two
+              const uint4 v = bt.a[d][mb][q >> 1];
+              const uint4 e0 = decode_bytes((q & 1) ? v.z : v.x, a_off), e1 = decode_bytes((q & 1) ? v.w : v.y, a_off);
+              af[mb] = make_uint4(__builtin_amdgcn_perm(e0.y, e0.x, 0x07060100u), __builtin_amdgcn_perm(e0.w, e0.z, 0x07060100u),
+                                  __builtin_amdgcn_perm(e1.y, e1.x, 0x07060100u), __builtin_amdgcn_perm(e1.w, e1.z, 0x07060100u));
+            }
           }
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             uint4 bf;
             if constexpr (BITS == 4) bf = decode_bytes(bt.w[d][j][q], w_off);
             else bf = decode_w<BITS, 6>(bt.w[d][j], q, w_off);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af),
-                                                             __builtin_bit_cast(bf16x8, bf), acc[j], 0, 0, 0);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+              acc[mb][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[mb]),
+                                                                   __builtin_bit_cast(bf16x8, bf), acc[mb][j], 0, 0, 0);
           }
         }
       }
     }
   };
 
-  // Epilogue operands of the item this thread will finish (item = tid when tid < 64*R).  They
+  // Epilogue operands of the item this thread will finish (item = tid when tid < 64*R*MB: row
+  // block tid / (64*R), row step (tid / 64) % R, accumulator lane tid % 64).  They
   // are requested BEFORE the stream, by every thread, without a branch (clamped indices, a
   // readable stand-in address for an absent operand) and stay untouched, as raw bits, until the
   // epilogue.  A wavefront's loads return in order: a use of one of these values before the main
   // loop - a conversion, or the register copy behind a value that is only loaded on one side of
   // a branch - waits for every weight load issued before it, and did: the wavefronts that own
   // an item used to start their table build only when their first weights had arrived.
-  const int ep_j = tid >> 6, ep_l = tid & 63;
+  const int ep_mb = (tid >> 6) / R, ep_j = (tid >> 6) % R, ep_l = tid & 63;
   const int64_t ep_n = n_base + 16 * ep_j + (ep_l & 15);
   const int64_t ep_nc = min(ep_n, g.N - 1);
   const bool has_bias = g.bias != nullptr, has_scale = !LATE && g.row_scale != nullptr;
@@ -215,7 +246,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   const float *scale_at = has_scale ? g.row_scale : g.w_cents;
   float ep_sc_raw[4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) ep_sc_raw[e] = scale_at[has_scale ? min(4 * (ep_l >> 4) + e, g.M - 1) : 0];
+  for (int e = 0; e < 4; ++e) ep_sc_raw[e] = scale_at[has_scale ? min(16 * ep_mb + 4 * (ep_l >> 4) + e, g.M - 1) : 0];
 
   // ---- then the packed stream ------------------------------------------------------
   // Batches in flight: two for the plain stream (decode of one overlaps the loads of the next);
@@ -284,15 +315,18 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   // ---- cross-wave sum in LDS (the tables are dead), fixed order ------------------------
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < R; ++j)
-    *reinterpret_cast<float4 *>(partial + ((wave * R + j) * 64 + lane) * 4) =
-        make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      *reinterpret_cast<float4 *>(partial + (((wave * MB + mb) * R + j) * 64 + lane) * 4) =
+          make_float4(acc[mb][j][0], acc[mb][j][1], acc[mb][j][2], acc[mb][j][3]);
   __syncthreads();
-  // accumulator e of lane l: token row 4*(l/16) + e, weight row l%16
-  if (tid < 64 * R && ep_n < g.N) {
-    float4 sum = *reinterpret_cast<const float4 *>(partial + ((0 * R + ep_j) * 64 + ep_l) * 4);
+  // accumulator e of lane l in row block mb: token row 16*mb + 4*(l/16) + e, weight row l%16
+  if (tid < 64 * R * MB && ep_n < g.N) {
+    const int ep_item = ep_mb * R + ep_j;
+    float4 sum = *reinterpret_cast<const float4 *>(partial + (ep_item * 64 + ep_l) * 4);
     for (int w = 1; w < WAVES; ++w) {
-      const float4 p = *reinterpret_cast<const float4 *>(partial + ((w * R + ep_j) * 64 + ep_l) * 4);
+      const float4 p = *reinterpret_cast<const float4 *>(partial + ((w * MB * R + ep_item) * 64 + ep_l) * 4);
       sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
     }
     const float v[4] = {sum.x, sum.y, sum.z, sum.w};
@@ -300,7 +334,7 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
     const float ep_bv = has_bias ? dyn_bits_to_f32(bias_size == 4 ? (ep_bias_lo | (ep_bias_hi << 16)) : ep_bias_lo, g.bias_dtype) : 0.0f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int m = 4 * (ep_l >> 4) + e;
+      const int m = 16 * ep_mb + 4 * (ep_l >> 4) + e;
       if (m >= g.M) continue;
       float sc = has_scale ? ep_sc_raw[e] : 1.0f;
       if constexpr (LATE) {  // produced by this launch: read where it is used

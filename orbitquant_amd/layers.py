@@ -14,7 +14,7 @@ the reference's `orbitquant::packed_linear_forward` does (layers.py:38-72,
 Inside the op (the reference's `_forward_impl`, layers.py:1079-1455, for AMD), one
 native call (`oq_quantized_linear`):
   1. fused rotate + per-token quantize (HIP) -> activation codes + token norms
-  2. packed-weight matmul (HIP): streaming kernel for <= 16 tokens, MFMA tile
+  2. packed-weight matmul (HIP): streaming kernel for <= 64 tokens, MFMA tile
      kernel otherwise.
 For a single token both run in ONE launch.  Shapes the code kernels do not take
 (activation widths above 4 bits with K not a multiple of 64 / 128) hand the matmul

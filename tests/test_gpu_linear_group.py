@@ -143,6 +143,29 @@ def test_few_token_launch_equals_rows_of_a_batch(dev, k, n, wbits):
         assert torch.equal(run(slice(2, 5)), batch[2:5])
 
 
+@pytest.mark.parametrize("k,n,wbits,abits", [(4096, 4096, 4, 4), (512, 14336, 3, 4), (14336, 4096, 4, 4), (2048, 9000, 2, 3),
+                                            (1024, 520, 6, 4), (512, 96, 8, 4), (1024, 4096, 4, 6), (4096, 600, 3, 6),
+                                            (512, 9000, 4, 8)])
+def test_seventeen_to_sixty_four_tokens_stream_like_sixteen(dev, k, n, wbits, abits):
+    """17 to 64 tokens take the streaming kernel with two or four blocks of sixteen token rows per
+    workgroup.  A token row's sums do not depend on the rows computed with it: every row of such a
+    launch equals the same row from launches of at most sixteen tokens, bit for bit."""
+    from orbitquant_amd import ops
+
+    c = make_group(dev, 64, k, [(n, wbits, True)], abits, torch.bfloat16, seed=700 + wbits + abits)
+    w = c["weights"][0]
+
+    def run(lo, hi):
+        return ops.packed_linear(c["codes"][lo:hi], c["norms"][lo:hi], c["cents"], w[0], w[1], w[2], code_format=c["fmt"],
+                                 activation_bits=abits, weight_bits=wbits, out_features=n, in_features=k, bias=w[5],
+                                 output_dtype=torch.bfloat16)
+
+    want = torch.cat([run(lo, lo + 16) for lo in range(0, 64, 16)])
+    assert torch.equal(run(0, 64), want)
+    for lo, hi in ((0, 17), (3, 35), (10, 42), (15, 64), (31, 64)):
+        assert torch.equal(run(lo, hi), want[lo:hi]), (lo, hi)
+
+
 WHOLE = [
     # one token, wide rows: quantizer launch, then the whole group in one launch
     dict(m=1, k=4096, shapes=[(4096, 2, False), (1024, 2, True), (1000, 3, False)], dtype=torch.bfloat16, block="paper"),
