@@ -156,6 +156,16 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
                               float *norms_out, void *stream);
 
 /*
+ * Sets (value != NULL) or clears one of the library's experiment switches, the OQ_* environment
+ * variables that pick a launch shape or turn a kernel variant off (OQ_GEMM_TILE, OQ_GEMM_WG_SPLIT,
+ * OQ_GEMV_CFG, OQ_NO_TOKEN_LINEAR, ...).  The library reads the environment once per process;
+ * tests and measurements that compare variants inside one process change a switch through this
+ * call.  Results stay correct under every setting; only which kernel computes them changes.
+ * Not thread-safe against running calls.  No counterpart in the reference.
+ */
+int oq_debug_override(const char *name, const char *value);
+
+/*
  * Packed-weight linear on quantized activations (the fused hot path):
  *
  *   out[m,n] = (sum_k c_a[code[m,k]] * c_w[idx[n,k]]) * s[m] * r_w[n] + bias[n]
@@ -165,7 +175,11 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
  * int8 surrogate.  M <= 64 takes the streaming small-M kernel (the weights are read and
  * decoded once, sixteen token rows per matrix instruction, up to four blocks of sixteen per
  * workgroup), larger M the MFMA tile kernel.  A token row's result does not depend on the
- * rows computed with it as long as the call stays within 64 rows.
+ * rows computed with it as long as the call stays within 64 rows.  A problem with few output
+ * tiles and many K-steps (some hundred tokens on a short-and-long matrix) is shared between
+ * workgroups along K: fp32 partial tiles go through a device buffer the library keeps per
+ * (device, stream) and grows on demand - the one allocation this entry point can make; it is
+ * skipped while the stream is being captured and inside oq_quantized_linear_static.
  *
  * codes        activation codes in code_format (see oq_rotate_quantize)
  * token_norms  fp32 [M]
@@ -276,8 +290,10 @@ int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_
 /*
  * oq_quantized_linear for callers that cannot allocate device memory or bring a workspace:
  * code running under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc.  No counterpart in the reference.  Same arguments and same results as
- * oq_quantized_linear, without the two scratch pointers: codes and norms pass through a buffer
+ * hipMalloc.  No counterpart in the reference.  Same arguments as oq_quantized_linear without
+ * the two scratch pointers, and the same results (except where oq_quantized_linear shares K
+ * between workgroups through a buffer of the library's own, see oq_packed_linear: this call
+ * never does, and the two then differ by the order of the last additions): codes and norms pass through a buffer
  * of OQ_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the library
  * runs on holds its own copy until the process ends).  The call allocates and frees nothing.
  * Shapes whose codes ([M, K/2] bytes for a_bits <= 4 and even K, else [M, K], rounded up to

@@ -19,7 +19,7 @@ OQ_VALUES_NONE, OQ_VALUES_SCALED, OQ_VALUES_UNIT_BF16 = 0, 1, 2
 _STATUS = {1: "invalid argument", 2: "unsupported", 3: "launch failure"}
 
 EXPORTS = (
-    "oq_device_ok", "oq_last_error", "oq_version", "oq_rotate_quantize", "oq_rotate_plan_bytes", "oq_rotate_plan_build", "oq_quantize_weight", "oq_rotate_quantize_mapped",
+    "oq_device_ok", "oq_last_error", "oq_version", "oq_debug_override", "oq_rotate_quantize", "oq_rotate_plan_bytes", "oq_rotate_plan_build", "oq_quantize_weight", "oq_rotate_quantize_mapped",
     "oq_packed_linear", "oq_packed_linear_group", "oq_packed_linear_mapped", "oq_quantized_linear", "oq_quantized_linear_group", "oq_quantized_linear_static", "oq_matmul_packed_weight", "oq_matmul_packed_adaln_int4", "oq_quantize_adaln_weight", "oq_unpack_lowbit", "oq_pack_lowbit",
     "oq_dequantize_packed_weight",
 )
@@ -57,6 +57,8 @@ def load() -> ctypes.CDLL:
     lib.oq_rotate_quantize_mapped.restype = c_int
     lib.oq_rotate_quantize_mapped.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f,
                                               vp, c_int, vp, c_int, vp, vp]
+    lib.oq_debug_override.restype = c_int
+    lib.oq_debug_override.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
     lib.oq_packed_linear.restype = c_int
     lib.oq_packed_linear.argtypes = [vp, c_int, vp, vp, c_int, vp, c_int, vp, vp, vp, c_int,
                                      c_i64, c_i64, c_i64, vp, c_int, vp]

@@ -37,6 +37,7 @@ SOURCES = {
     "packed_gemm_bytes.hip": [],
     "packed_gemm_tiled.hip": [],
     "packed_gemm_staged.hip": [],
+    "packed_gemm_splitk.hip": [],
     "packed_gemm_av.hip": [],
     "packed_gemv.hip": [],
     "packed_gemv_group.hip": [],

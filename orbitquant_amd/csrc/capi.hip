@@ -49,14 +49,45 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
   return true;
 }
 
-const char *debug_env(int which) {
-  static const char *const names[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES", "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE", "OQ_GEMV_MAX_M"};
-  static const char *values[ENV_COUNT];
+namespace {
+const char *const kEnvNames[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES",
+                                          "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE",
+                                          "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT"};
+const char *env_values[ENV_COUNT];
+void env_load() {
   static std::once_flag once;
   std::call_once(once, [] {
-    for (int i = 0; i < ENV_COUNT; ++i) values[i] = getenv(names[i]);
+    for (int i = 0; i < ENV_COUNT; ++i) env_values[i] = getenv(kEnvNames[i]);
   });
-  return values[which];
+}
+}  // namespace
+
+namespace {
+thread_local int no_allocation_depth = 0;
+struct NoAllocation {
+  NoAllocation() { ++no_allocation_depth; }
+  ~NoAllocation() { --no_allocation_depth; }
+};
+}  // namespace
+
+bool allocation_forbidden() { return no_allocation_depth > 0; }
+
+// The experiment switches: read from the environment once per process, then only changed through
+// oq_debug_override.
+const char *debug_env(int which) {
+  env_load();
+  return env_values[which];
+}
+
+int debug_env_set(const char *name, const char *value) {
+  env_load();
+  for (int i = 0; i < ENV_COUNT; ++i) {
+    if (strcmp(name, kEnvNames[i]) == 0) {
+      env_values[i] = value != nullptr ? strdup(value) : nullptr;  // a few bytes per call, never freed: readers may hold the old one
+      return OQ_OK;
+    }
+  }
+  return fail(OQ_ERR_INVALID, "debug_override: unknown switch %s", name);
 }
 
 // kernels (defined in the other translation units)
@@ -252,6 +283,11 @@ static int packed_linear_impl(const void *codes, int code_format, const float *t
   return apply_value_map(out, M * N, out_map, s);
 }
 
+int oq_debug_override(const char *name, const char *value) {
+  if (name == nullptr) return fail(OQ_ERR_INVALID, "debug_override: null name");
+  return debug_env_set(name, value);
+}
+
 int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
                      int a_bits, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                      const float *w_centroids, const void *bias, int bias_dtype, int64_t M, int64_t N,
@@ -381,6 +417,7 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
                 (long long)M, (long long)K, (unsigned long long)(norms_at + 4u * static_cast<uint64_t>(M)), kStaticScratchBytes);
   unsigned char *base = nullptr;
   if (int rc = static_scratch_address(&base)) return rc;
+  NoAllocation guard;  // no launch shape that wants a buffer of the library's own
   return oq_quantized_linear(x, x_dtype, input_map, M, K, perm, signs, boundaries, act_centroids, a_bits, block, eps,
                              inv_sqrt_block, rotate_plan, packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, N, base,
                              reinterpret_cast<float *>(base + norms_at), out, out_dtype, output_map, stream);

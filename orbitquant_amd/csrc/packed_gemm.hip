@@ -13,7 +13,7 @@ int gemm_launch_bytes(const GemmArgs &g, int bits, int tile, hipStream_t stream)
 // constants are microseconds measured on an MI355X: the "busy" set for launches long enough
 // to run at sustained clocks with every CU occupied, the other for short launches; weight
 // widths other than 4 pay for their longer index extraction, least on the largest tile.
-int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits) {
+static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, double *cost_out) {
   const bool can_split = K % 256 == 0;  // a quarter of the K-steps per wavefront
   const char *force = debug_env(ENV_GEMM_TILE);
   if (force != nullptr && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
@@ -45,7 +45,55 @@ int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits) {
     const int64_t tiles = ((M + 127) / 128) * ((N + 95) / 96);
     const double per_step = (busy ? shapes[3].step_busy : shapes[3].step_short) * (bits == 4 ? 1.0 : shapes[3].other_bits);
     const double cost = static_cast<double>((tiles + 255) / 256) * (7.5 + steps / 4.0 * per_step);
-    if (cost < best_cost) best = 4;
+    if (cost < best_cost) {
+      best = 4;
+      best_cost = cost;
+    }
+  }
+  if (cost_out != nullptr) *cost_out = best_cost;
+  return best;
+}
+
+int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits) { return choose_tile_with_cost(M, N, K, bits, nullptr); }
+
+int gemm_splitk_reduce(const float *partials, int splits, int64_t M, int64_t N, const float *row_scale,
+                       const uint16_t *row_norms, const void *bias, int bias_dtype, void *out, int out_dtype,
+                       hipStream_t stream);  // packed_gemm_splitk.hip
+int apply_value_map(void *out, int64_t count, const uint16_t *table, hipStream_t stream);
+
+// Short-and-long problems at a few hundred tokens (128 x 4096 outputs over K = 14336) have a few dozen tiles
+// for 256 CUs, each with hundreds of K-steps.  Such a launch shares K between workgroups: `splits`
+// workgroups per 128x128 tile, each over its part of the K-steps, raw fp32 partial tiles into a buffer, and a
+// small second launch that adds them in order and applies the epilogue.  Returns the number of parts (1:
+// none), chosen with the cost model above plus the second launch (3 us and the partial tiles, written and
+// read back, at 3 TB/s):
+// every part keeps at least sixteen K-steps, the partial tiles stay within 64 MB, and the split has to
+// promise 15 % over the best single launch.  OQ_GEMM_WG_SPLIT overrides (1 = never).
+int gemm_choose_splits(int64_t M, int64_t N, int64_t K, int bits) {
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128), steps = K / 64;
+  auto allowed = [&](int s) { return s >= 2 && s <= 8 && steps / s >= 16 && M * N * 4 * s <= (64ll << 20); };
+  if (const char *force = debug_env(ENV_GEMM_WG_SPLIT)) {
+    int s = atoi(force);
+    while (s > 1 && !allowed(s)) --s;
+    return s < 1 ? 1 : s;
+  }
+  if (debug_env(ENV_GEMM_TILE) != nullptr) return 1;  // a forced tile is a forced single launch
+  double single = 0.0;
+  choose_tile_with_cost(M, N, K, bits, &single);
+  const double width = bits == 4 ? 1.0 : 1.28;
+  int best = 1;
+  double best_cost = 0.85 * single;
+  for (int s = 2; s <= 8; ++s) {
+    if (!allowed(s)) continue;
+    const int64_t groups = tiles * s;
+    const double per_step = (groups <= 256 ? 0.5 : 0.8) * width;
+    const double rounds = static_cast<double>((groups + 511) / 512);
+    const double cost = rounds * (4.5 + static_cast<double>(steps / s) * per_step) + 3.0 +
+                        static_cast<double>(M) * static_cast<double>(N) * (8.0 * s + 2.0) / 3.0e6;  // partial tiles written, then read
+    if (cost < best_cost) {
+      best = s;
+      best_cost = cost;
+    }
   }
   return best;
 }
@@ -64,10 +112,25 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
   g.out_map = OutMap{out_map, out_map != nullptr && out_dtype == OQ_BF16 ? kWideLoBf16 : -1};
-  const int tile = gemm_choose_tile(M, N, K, bits);
-  if (a_mode == A_NIBBLE) return launch_mode<A_NIBBLE>(g, bits, tile, stream);
-  if (a_mode == A_U8) return gemm_launch_bytes(g, bits, tile, stream);
-  return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
+  int tile = gemm_choose_tile(M, N, K, bits);
+  if (a_mode != A_NIBBLE && a_mode != A_U8) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
+  g.k_splits = 1;
+  const int splits = gemm_choose_splits(M, N, K, bits);
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (splits > 1 && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
+    // (not while the stream is being captured: the buffer may have to grow)
+    float *partials = static_cast<float *>(stream_workspace(static_cast<size_t>(M) * N * 4 * splits, stream));
+    if (partials != nullptr) {
+      g.k_splits = splits;
+      g.partials = partials;
+      tile = 0;  // 128x128 tiles, two workgroups per CU
+    }
+  }
+  const int rc = a_mode == A_NIBBLE ? launch_mode<A_NIBBLE>(g, bits, tile, stream) : gemm_launch_bytes(g, bits, tile, stream);
+  if (rc != OQ_OK || g.k_splits == 1) return rc;
+  if (int rc2 = gemm_splitk_reduce(g.partials, g.k_splits, M, N, row_scale, row_norms, bias, bias_dtype, out, out_dtype, stream))
+    return rc2;
+  return out_map == nullptr ? OQ_OK : apply_value_map(out, M * N, out_map, stream);
 }
 
 }  // namespace oq

@@ -67,7 +67,14 @@ struct GemmArgs {
   int out_dtype;
   OutMap out_map;            // optional elementwise function of the outputs (gemm_epilogue.h)
   int tiles_m, tiles_n;
+  // K shared between workgroups (grid.y = k_splits > 1; code activations, KSPLIT = 1 only): every
+  // workgroup writes its raw fp32 partial tile to partials[blockIdx.y][M][N]; packed_gemm_splitk.hip
+  // adds them up and applies the epilogue.
+  int k_splits;
+  float *partials;
 };
+
+void *stream_workspace(size_t bytes, hipStream_t stream);  // packed_gemm_tiled.hip
 
 namespace {
 
@@ -155,7 +162,18 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // packed operands of NBUF consecutive K-steps
   uint4 pa[NBUF][FM][kAVec];
   uint32_t pw[NBUF][FN][BITS];
-  const int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
+  int steps = static_cast<int>(g.K / 64) / KSPLIT;  // K-steps of this wavefront
+  if constexpr (KSPLIT == 1 && (AM == A_NIBBLE || AM == A_U8)) {
+    if (g.k_splits > 1) {  // this workgroup's share of the K-steps
+      const int z = blockIdx.y;
+      const int first = static_cast<int>(static_cast<int64_t>(steps) * z / g.k_splits);
+      steps = static_cast<int>(static_cast<int64_t>(steps) * (z + 1) / g.k_splits) - first;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(first) * kAStep;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) wp[j] += static_cast<int64_t>(first) * (8 * BITS);
+    }
+  }
   if constexpr (KSPLIT > 1) {
 #pragma unroll
     for (int i = 0; i < FM; ++i) ap[i] += static_cast<int64_t>(wave) * steps * kAStep;  // (A_STAGED: every ap[i] is the same base)
@@ -340,9 +358,21 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 
   __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused from here on
   if constexpr (KSPLIT == 1) {
+    void *out = g.out;
+    int out_dtype = g.out_dtype;
+    OutMap out_map = g.out_map;
+    if (g.k_splits > 1) {  // raw partial sums: factors of one, no bias, fp32 (x * 1 * 1 + 0 is x)
+      epi.rn = 1.0f;
+      epi.bv = 0.0f;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) epi.sc[i] = 1.0f;
+      out = g.partials + static_cast<int64_t>(blockIdx.y) * g.M * g.N;
+      out_dtype = OQ_F32;
+      out_map = OutMap{nullptr, -1};
+    }
     gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, wn, TN, tid, g.M, g.N,
-                          g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out, g.out_dtype,
-                          reinterpret_cast<unsigned char *>(lds), g.out_map);
+                          g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, out, out_dtype,
+                          reinterpret_cast<unsigned char *>(lds), out_map);
   } else {
     // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
     // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
@@ -414,7 +444,9 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   const int64_t total = static_cast<int64_t>(g.tiles_m) * g.tiles_n;
   if (total > 0x7fffffffLL) return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: too many tiles");
   auto kern = packed_gemm_kernel<AM, BITS, FM, FN, KSPLIT>;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total)), dim3(256), 0, stream, g);
+  const unsigned splits = (KSPLIT == 1 && (AM == A_NIBBLE || AM == A_U8) && g.k_splits > 1) ? static_cast<unsigned>(g.k_splits) : 1u;
+  if (splits == 1) g.k_splits = 1;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), 0, stream, g);
   return check_launch("packed_gemm");
 }
 

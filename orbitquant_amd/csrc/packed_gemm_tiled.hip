@@ -35,14 +35,30 @@ __global__ __launch_bounds__(256) void tile_activations_kernel(const uint16_t *x
 
 // The operand-order copy lives in a buffer the library keeps per (device, stream) and grows on demand: calls on one
 // stream are ordered, so they can share it; it is released when the process ends.
+template <int BITS>
+int launch_tiled(const GemmArgs &g, int tile, hipStream_t stream) {
+  if (tile == 4) return launch_cfg<A_TILED, BITS, 4, 3, 4>(g, stream);
+  if (tile == 3) return launch_cfg<A_TILED, BITS, 4, 3>(g, stream);
+  if (tile == 1 || tile == 2) return launch_cfg<A_TILED, BITS, 2, 4>(g, stream);
+  return launch_cfg<A_TILED, BITS, 2, 2>(g, stream);
+}
+
+}  // namespace
+
+// A device buffer per (device, stream), grown on demand and kept: work on one stream is ordered, so
+// a later call may reuse what an earlier one has finished with.  NULL when it cannot be had.
+namespace {
 struct Workspace {
   void *ptr = nullptr;
   size_t bytes = 0;
 };
 
+}  // namespace
+
 void *stream_workspace(size_t bytes, hipStream_t stream) {
   static std::mutex lock;
   static std::map<std::pair<int, hipStream_t>, Workspace> spaces;
+  if (allocation_forbidden()) return nullptr;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> guard(lock);
@@ -60,16 +76,6 @@ void *stream_workspace(size_t bytes, hipStream_t stream) {
   w.bytes = want;
   return w.ptr;
 }
-
-template <int BITS>
-int launch_tiled(const GemmArgs &g, int tile, hipStream_t stream) {
-  if (tile == 4) return launch_cfg<A_TILED, BITS, 4, 3, 4>(g, stream);
-  if (tile == 3) return launch_cfg<A_TILED, BITS, 4, 3>(g, stream);
-  if (tile == 1 || tile == 2) return launch_cfg<A_TILED, BITS, 2, 4>(g, stream);
-  return launch_cfg<A_TILED, BITS, 2, 2>(g, stream);
-}
-
-}  // namespace
 
 int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits);  // packed_gemm.hip
 

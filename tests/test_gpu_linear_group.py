@@ -99,23 +99,14 @@ def test_group_equals_one_call_per_matrix(dev, case, dtype):
 
 
 @pytest.mark.parametrize("rows_per_step", ["1", "2", "4"])
-def test_group_result_does_not_depend_on_rows_per_workgroup(dev, rows_per_step):
-    """The launch shape is a speed choice only.  (The override is read once per process, so this test
-    runs its three cases in child processes.)"""
-    import os
-    import subprocess
-    import sys
-
-    code = (
-        "import sys, torch; sys.path.insert(0, 'tests'); import test_gpu_linear_group as t\n"
-        "dev = torch.device('cuda:0')\n"
-        "c = t.make_group(dev, 3, 2048, [(1000, 2, False), (520, 3, True), (4096, 4, False)], 4, torch.bfloat16, seed=7)\n"
-        "assert all(torch.equal(a, b) for a, b in zip(t.grouped(c), t.one_by_one(c)))\n"
-        "print('same')\n")
-    env = dict(os.environ, OQ_GEMV_GROUP_R=rows_per_step)
-    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110,
-                          cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    assert done.returncode == 0 and "same" in done.stdout, done.stderr[-2000:]
+def test_group_result_does_not_depend_on_rows_per_workgroup(dev, rows_per_step, library_switch):
+    """The launch shape is a speed choice only."""
+    c = make_group(dev, 3, 2048, [(1000, 2, False), (520, 3, True), (4096, 4, False)], 4, torch.bfloat16, seed=7)
+    want = one_by_one(c)
+    library_switch("OQ_GEMV_GROUP_R", rows_per_step)
+    assert all(torch.equal(a, b) for a, b in zip(grouped(c), want))
+    library_switch("OQ_NO_GEMV_GROUP", "1")          # and with the single launch switched off
+    assert all(torch.equal(a, b) for a, b in zip(grouped(c), want))
 
 
 @pytest.mark.parametrize("k,n,wbits", [(4096, 4096, 4), (4096, 14336, 3), (2048, 520, 2), (14336, 4096, 4), (1024, 96, 6),

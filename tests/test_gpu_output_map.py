@@ -68,11 +68,11 @@ CASES = [
 
 @pytest.mark.parametrize(("m", "k", "n", "wbits", "abits", "dtype", "tile"), CASES)
 @pytest.mark.parametrize("fn", [gelu, torch.nn.functional.silu])
-def test_output_map_equals_function_of_plain_output(dev, m, k, n, wbits, abits, dtype, tile, fn, monkeypatch):
+def test_output_map_equals_function_of_plain_output(dev, m, k, n, wbits, abits, dtype, tile, fn, library_switch):
     from orbitquant_amd import ops
 
     if tile is not None:
-        monkeypatch.setenv("OQ_GEMM_TILE", tile)
+        library_switch("OQ_GEMM_TILE", tile)
     c = make_case(dev, m, k, n, wbits, abits, dtype, seed=m + k + n)
     table = ops.activation_table(fn, dtype, dev)
     plain = linear(c)

@@ -295,9 +295,9 @@ def test_packed_linear_tile_kernel(dev, m, n, k, wbits, abits, block, with_bias,
     (300, 200, 1024, 4, 6), (130, 96, 256, 4, 8), (257, 384, 1536, 3, 6), (64, 64, 64, 2, 5), (100, 136, 512, 6, 6),
     (90, 72, 384, 8, 8), (515, 520, 1152, 4, 4)])
 @pytest.mark.parametrize("tile", ["0", "1", "3"])
-def test_packed_linear_byte_codes_tile_kernel(dev, m, n, k, wbits, abits, tile, monkeypatch):
+def test_packed_linear_byte_codes_tile_kernel(dev, m, n, k, wbits, abits, tile, library_switch):
     """One activation code per byte (a_bits up to 8) through the all-table tile kernel."""
-    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+    library_switch("OQ_GEMM_TILE", tile)
     rng = np.random.default_rng(m + 3 * n + k + wbits + abits + int(tile))
     layer = make_layer(rng, n, k, wbits, abits)
     _, x32 = make_x(rng, m, k, torch.bfloat16)
@@ -311,8 +311,8 @@ def test_packed_linear_byte_codes_tile_kernel(dev, m, n, k, wbits, abits, tile, 
 
 
 @pytest.mark.parametrize("tile", ["0", "1", "2", "3"])
-def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
-    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+def test_packed_linear_every_tile_shape(dev, tile, library_switch):
+    library_switch("OQ_GEMM_TILE", tile)
     rng = np.random.default_rng(int(tile) + 50)
     m, n, k = 515, 520, 1152
     layer = make_layer(rng, n, k, 4, 4)
@@ -325,9 +325,9 @@ def test_packed_linear_every_tile_shape(dev, tile, monkeypatch):
 
 @pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4"])
 @pytest.mark.parametrize(("m", "n", "k"), [(17, 8, 256), (33, 24, 512), (300, 8, 256)])
-def test_packed_linear_tiny_outputs_every_tile(dev, m, n, k, tile, monkeypatch):
+def test_packed_linear_tiny_outputs_every_tile(dev, m, n, k, tile, library_switch):
     """Outputs much smaller than a tile: every row / column clamp and store guard is exercised."""
-    monkeypatch.setenv("OQ_GEMM_TILE", tile)
+    library_switch("OQ_GEMM_TILE", tile)
     rng = np.random.default_rng(m * 5 + n + k + int(tile))
     layer = make_layer(rng, n, k, 4, 4)
     _, x32 = make_x(rng, m, k, torch.bfloat16)
@@ -338,9 +338,9 @@ def test_packed_linear_tiny_outputs_every_tile(dev, m, n, k, tile, monkeypatch):
 
 
 @pytest.mark.parametrize(("m", "n", "k", "wbits"), [(300, 200, 1024, 4), (128, 96, 256, 4), (515, 1152, 2304, 3), (130, 104, 512, 6)])
-def test_packed_linear_k_split_kernel(dev, m, n, k, wbits, monkeypatch):
+def test_packed_linear_k_split_kernel(dev, m, n, k, wbits, library_switch):
     """Four wavefronts share one output tile and a quarter of K each; partial tiles are summed through LDS."""
-    monkeypatch.setenv("OQ_GEMM_TILE", "4")
+    library_switch("OQ_GEMM_TILE", "4")
     rng = np.random.default_rng(m + n + k)
     layer = make_layer(rng, n, k, wbits, 4)
     _, x32 = make_x(rng, m, k, torch.bfloat16)
@@ -350,6 +350,44 @@ def test_packed_linear_k_split_kernel(dev, m, n, k, wbits, monkeypatch):
     check_outputs(got, want, s, layer["r"].float().numpy(), k, "k-split")
     again = run_packed_linear(dev, layer, codes, s, "nibble")
     assert torch.equal(got, again)  # fixed summation order: bitwise reproducible
+
+
+@pytest.mark.parametrize(("m", "n", "k", "wbits", "abits", "splits"), [
+    (128, 256, 2048, 4, 4, 2), (65, 520, 4096, 4, 4, 4), (300, 136, 8192, 3, 3, 8), (129, 96, 4608, 2, 4, 3),
+    (200, 264, 3072, 6, 4, 2), (130, 128, 2048, 8, 4, 2), (256, 384, 4096, 4, 6, 4), (100, 72, 2048, 3, 8, 2)])
+def test_packed_linear_k_shared_between_workgroups(dev, m, n, k, wbits, abits, splits, library_switch):
+    """Several workgroups per output tile, each over a part of K, fp32 partial tiles added by a second launch:
+    against the oracle, against the single launch (same products, another summation order), and reproducible."""
+    rng = np.random.default_rng(m + n + k + wbits)
+    layer = make_layer(rng, n, k, wbits, abits)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    x32[2] = 0
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    fmt = "nibble" if abits <= 4 else "u8"
+    want = oracle_linear(layer, codes, s, torch.bfloat16)
+    library_switch("OQ_GEMM_WG_SPLIT", "1")
+    single = run_packed_linear(dev, layer, codes, s, fmt)
+    library_switch("OQ_GEMM_WG_SPLIT", str(splits))
+    got = run_packed_linear(dev, layer, codes, s, fmt)
+    check_outputs(got, want, s, layer["r"].float().numpy(), k, f"{splits} parts of K")
+    assert torch.equal(got, run_packed_linear(dev, layer, codes, s, fmt))   # fixed order of the parts
+    scale = single.float().abs().max().item()
+    assert (got.float() - single.float()).abs().max().item() <= scale * 2.0 ** -7
+    zero_row = got[2].float().cpu().numpy()      # a zero token gives exactly the bias
+    assert np.array_equal(zero_row, torch.from_numpy(layer["bias"]).to(torch.bfloat16).float().numpy())
+    fp32 = run_packed_linear(dev, layer, codes, s, fmt, torch.float32)
+    check_outputs(fp32, oracle_linear(layer, codes, s, torch.float32), s, layer["r"].float().numpy(), k, "fp32 out")
+
+
+def test_packed_linear_chooses_shared_k_for_short_and_long_problems(dev):
+    """The dispatcher's own choice on a short-and-long problem (few tiles, many K-steps) against the oracle."""
+    rng = np.random.default_rng(77)
+    m, n, k = 128, 512, 14336
+    layer = make_layer(rng, n, k, 4, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    got = run_packed_linear(dev, layer, codes, s, "nibble")
+    check_outputs(got, oracle_linear(layer, codes, s, torch.bfloat16), s, layer["r"].float().numpy(), k, "dispatcher's choice")
 
 
 @pytest.mark.parametrize("m", [1, 4, 16, 3])
@@ -586,10 +624,13 @@ def test_dropin_matmul_packed_weight_rows_1536(dev):
 
 @pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
 @pytest.mark.parametrize(("m", "n", "k"), [(300, 200, 256), (512, 1152, 4608), (257, 96, 64), (2048, 384, 1152)])
-def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k):
+def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k, library_switch):
     """bf16 activations at M >= 256 take the operand-order pass + tile kernel: against the oracle, and
-    bit for bit against the code kernel fed with the codes whose centroids are those activations."""
+    bit for bit against the code kernel fed with the codes whose centroids are those activations (both as
+    one launch over all of K: the code kernel would share K between workgroups on some of these shapes)."""
     from orbitquant_amd import ops
+
+    library_switch("OQ_GEMM_WG_SPLIT", "1")
 
     rng = np.random.default_rng(bits * 7 + m)
     layer = make_layer(rng, n, k, bits, 4)

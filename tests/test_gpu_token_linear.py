@@ -73,13 +73,13 @@ ONE_TOKEN = [
 
 
 @pytest.mark.parametrize(("k", "n", "wbits", "abits", "dtype", "block", "with_bias"), ONE_TOKEN)
-def test_one_token_single_launch_equals_two_launches(dev, k, n, wbits, abits, dtype, block, with_bias, monkeypatch):
+def test_one_token_single_launch_equals_two_launches(dev, k, n, wbits, abits, dtype, block, with_bias, library_switch):
     c = make_case(dev, 1, k, n, wbits, abits, dtype, block, with_bias, seed=k + n + wbits)
     want = two_calls(c)
     got = one_call(c)
     assert torch.equal(got, want)
     # and the switch that forces the two-launch route inside the same entry point
-    monkeypatch.setenv("OQ_NO_TOKEN_LINEAR", "1")
+    library_switch("OQ_NO_TOKEN_LINEAR", "1")
     assert torch.equal(one_call(c), want)
 
 

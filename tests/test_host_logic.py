@@ -33,6 +33,18 @@ def test_library_exports_every_symbol_the_header_declares():
     assert loaded.oq_version().decode().startswith("orbitquant-hip")
 
 
+def test_debug_override_knows_its_switches():
+    """oq_debug_override touches no GPU: known switches are accepted (and cleared again), others refused."""
+    from orbitquant_amd import _lib
+
+    lib = _lib.load()
+    for name in (b"OQ_GEMM_TILE", b"OQ_GEMM_WG_SPLIT", b"OQ_GEMV_CFG", b"OQ_NO_TOKEN_LINEAR", b"OQ_GEMV_MAX_M"):
+        assert lib.oq_debug_override(name, b"1") == 0
+        assert lib.oq_debug_override(name, None) == 0
+    assert lib.oq_debug_override(b"OQ_NO_SUCH_SWITCH", b"1") != 0 and b"unknown switch" in lib.oq_last_error()
+    assert lib.oq_debug_override(None, b"1") != 0
+
+
 def test_product_codebooks_match_reference_generated_fixture(golden_dir):
     from orbitquant_amd.codebooks import get_codebook
 

@@ -80,6 +80,7 @@ def call(layer, x, *, static):
     (4096, 512, 3, 6, torch.bfloat16, (40, 24)),     # one code per byte (six-bit activations)
     (3072, 256, 2, 3, torch.float16, (33, 1)),       # two launches, then the single launch of one token
     (1152, 128, 4, 4, torch.float32, (20, 3)),
+    (4096, 256, 4, 4, torch.bfloat16, (128, 64)),    # few tiles, many K-steps: the allocating call shares K between workgroups
 ])
 def test_static_scratch_equals_caller_scratch(dev, k, n, wbits, abits, dtype, sizes):
     layer = make_layer(dev, k, n, wbits, abits, dtype, seed=k + n)
@@ -89,11 +90,18 @@ def test_static_scratch_equals_caller_scratch(dev, k, n, wbits, abits, dtype, si
         rc, got = call(layer, x, static=True)
         assert rc_ref == 0 and rc == 0
         assert not torch.isnan(got.float()).any()
+        if k == 4096 and m == 128:
+            # the call that may allocate adds partial sums of K from a buffer of the library's own; the static call
+            # never takes one: same products, another order of the last additions
+            assert (got.float() - want.float()).abs().max().item() <= want.float().abs().max().item() * 2.0 ** -7
+            continue
         assert torch.equal(got, want), f"m={m}: {(got.float() - want.float()).abs().max().item()}"
 
 
-def test_static_scratch_fills_to_its_limit_and_refuses_beyond(dev):
+def test_static_scratch_fills_to_its_limit_and_refuses_beyond(dev, library_switch):
     from orbitquant_amd import _lib
+
+    library_switch("OQ_GEMM_WG_SPLIT", "1")   # the allocating call as one launch over K, like the static one
 
     lib = _lib.load()
     k = 4096
