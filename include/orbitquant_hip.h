@@ -322,7 +322,7 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
  * Replaces matmul_packed_weight (torch_binding.cpp:7-12,32-38; packed_matmul.cu:1335-1713).
  * bits in [1, 8].  token_scale: NULL, or fp32 [M] multiplied into row m (lets the
  * caller pass unit-norm bf16 centroids plus token norms).
- * The one entry point that keeps device memory of its own: bf16 activations with M >= 256 are first
+ * Keeps device memory of its own: bf16 activations (from two tokens on; one token on large matrices) are first
  * rewritten into the matrix core's operand order, into a buffer of 2 * M * K bytes (rows padded to 32)
  * that the library keeps per (device, stream), grows when a larger call comes and releases when the
  * process ends.  Calls on one stream are ordered and share it; while the stream is being captured

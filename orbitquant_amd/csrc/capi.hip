@@ -52,7 +52,7 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
 namespace {
 const char *const kEnvNames[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES",
                                           "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE",
-                                          "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT"};
+                                          "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT", "OQ_FLOAT_GEMM_MIN_M"};
 const char *env_values[ENV_COUNT];
 void env_load() {
   static std::once_flag once;
@@ -431,7 +431,13 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   if (M == 0) return OQ_OK;
   if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
   hipStream_t s = as_stream(stream);
-  if (x_dtype == OQ_BF16 && M >= 256 && K % 64 == 0 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) &&
+  // bf16 activations take the tile kernel from two tokens on (one token on large matrices): measured against
+  // the float-activation kernels below it is 3-4 times faster from 9 to 255 tokens (4096x4096 W4: 104 -> 28 us)
+  // and up to 13 times at 2 to 8; only a single token on a small matrix is 2-3 us quicker on the
+  // shape-agnostic kernel.  OQ_FLOAT_GEMM_MIN_M overrides, for measurements.
+  int64_t tile_kernel_from = N * K >= (int64_t{32} << 20) ? 1 : 2;
+  if (const char *v = debug_env(ENV_FLOAT_GEMM_MIN_M)) tile_kernel_from = atoi(v) > 1 ? atoi(v) : 1;
+  if (x_dtype == OQ_BF16 && M >= tile_kernel_from && K % 64 == 0 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) &&
       gemm_supported(K, bits)) {
     // Large M: the tile kernel of the code path on activation values.  Either one pass first puts the activations
     // into the matrix core's operand order (fastest on large problems; needs a buffer, so not while the stream is

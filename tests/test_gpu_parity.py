@@ -625,7 +625,7 @@ def test_dropin_matmul_packed_weight_rows_1536(dev):
 @pytest.mark.parametrize("bits", [2, 3, 4, 6, 8])
 @pytest.mark.parametrize(("m", "n", "k"), [(300, 200, 256), (512, 1152, 4608), (257, 96, 64), (2048, 384, 1152)])
 def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k, library_switch):
-    """bf16 activations at M >= 256 take the operand-order pass + tile kernel: against the oracle, and
+    """bf16 activations take the operand-order pass + tile kernel: against the oracle, and
     bit for bit against the code kernel fed with the codes whose centroids are those activations (both as
     one launch over all of K: the code kernel would share K between workgroups on some of these shapes)."""
     from orbitquant_amd import ops
