@@ -137,10 +137,15 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
   // all the parallelism it needs; with at most sixteen rows it wins only when a row has several units (K = 14336
   // in blocks of 2048, one token: 7.9 us against 10.1 us; K = 1152: 3.8 against 4.4) and loses when the row is one
   // block (K = 4096 = one block: 9.9 against 5.6 us), which the kernel below spreads over a whole workgroup.
+  // A wavefront alone on a block of 2048 or 4096 values takes 7.5 / 10.4 us whatever the number of rows, the
+  // workgroup-per-row kernel 6-7 us: up to 512 rows (every row's workgroup has a CU to itself or shares it with
+  // one other) rows of one or two such blocks stay with the kernel below too (K = 4096 = one block, 17 to 512
+  // rows: 10.3-11.3 against 6.9-9.6 us; from 1024 rows on the plan kernel is level or ahead).
   int64_t fast_min_m = 17;
-  if (const char *v = debug_env(ENV_RQ_FAST_MIN_M)) fast_min_m = atoi(v);
   const int64_t unit = block > 512 ? block : 512;
   const bool several_units = (K + unit - 1) / unit >= 3;
+  if (block >= 2048 && !several_units) fast_min_m = 513;
+  if (const char *v = debug_env(ENV_RQ_FAST_MIN_M)) fast_min_m = atoi(v);
   if (plan != nullptr && input_map == nullptr && (M >= fast_min_m || several_units)) {
     RqArgs checked;
     bool vec_checked = false;
