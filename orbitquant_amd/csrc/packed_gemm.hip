@@ -22,7 +22,7 @@ static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, doub
   static const Shape shapes[4] = {{128, 128, 4.5, 0.8, 1.19, 1.28}, {128, 256, 5.5, 1.0, 1.0, 1.34},
                                   {256, 256, 7.0, 1.5, 1.68, 1.13}, {256, 192, 6.0, 1.15, 1.24, 1.30}};
   const double steps = static_cast<double>(K / 64);
-  const bool busy = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) > 2.0e11;
+  const bool busy = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) > 5.0e10;  // some 50 us of work
   int best = 0;
   double best_cost = 0.0;
   for (int t = 0; t < 4; ++t) {
