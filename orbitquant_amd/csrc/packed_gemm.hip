@@ -13,14 +13,16 @@ int gemm_launch_bytes(const GemmArgs &g, int bits, int tile, hipStream_t stream)
 // constants are microseconds measured on an MI355X: the "busy" set for launches long enough
 // to run at sustained clocks with every CU occupied, the other for short launches; weight
 // widths other than 4 pay for their longer index extraction, least on the largest tile.
-static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, double *cost_out) {
+// byte_codes: one activation code per byte (eight single lookups per operand instead of four pair lookups);
+// a K-step then costs 1.07-1.23 times as much, least on the tiles with many columns per activation row.
+static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, double *cost_out, bool byte_codes = false) {
   const bool can_split = K % 256 == 0;  // a quarter of the K-steps per wavefront
   const char *force = debug_env(ENV_GEMM_TILE);
   if (force != nullptr && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
   if (force != nullptr && force[0] == '4' && can_split) return 4;
-  struct Shape { int tm, tn; double fixed, step_short, step_busy, other_bits; };
-  static const Shape shapes[4] = {{128, 128, 4.5, 0.8, 1.19, 1.28}, {128, 256, 5.5, 1.0, 1.0, 1.34},
-                                  {256, 256, 7.0, 1.5, 1.68, 1.13}, {256, 192, 6.0, 1.15, 1.24, 1.30}};
+  struct Shape { int tm, tn; double fixed, step_short, step_busy, other_bits, bytes; };
+  static const Shape shapes[4] = {{128, 128, 4.5, 0.8, 1.19, 1.28, 1.20}, {128, 256, 5.5, 1.0, 1.0, 1.34, 1.07},
+                                  {256, 256, 7.0, 1.5, 1.68, 1.13, 1.10}, {256, 192, 6.0, 1.15, 1.24, 1.30, 1.23}};
   const double steps = static_cast<double>(K / 64);
   const bool busy = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) > 5.0e10;  // some 50 us of work
   int best = 0;
@@ -29,7 +31,7 @@ static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, doub
     const Shape &sh = shapes[t];
     const int64_t tiles = ((M + sh.tm - 1) / sh.tm) * ((N + sh.tn - 1) / sh.tn);
     const int64_t capacity = t == 0 ? 512 : 256;
-    const double width = bits == 4 ? 1.0 : sh.other_bits;
+    const double width = (bits == 4 ? 1.0 : sh.other_bits) * (byte_codes ? sh.bytes : 1.0);
     const double per_step = (busy ? sh.step_busy : sh.step_short) * width;
     const int64_t full = tiles / capacity, rest = tiles % capacity;
     // a 128x128 workgroup alone on its CU has the LDS to itself
@@ -43,7 +45,8 @@ static int choose_tile_with_cost(int64_t M, int64_t N, int64_t K, int bits, doub
   }
   if (can_split) {  // 128x96 tiles, four wavefronts share the K range (+ about 1.5 us of reduction)
     const int64_t tiles = ((M + 127) / 128) * ((N + 95) / 96);
-    const double per_step = (busy ? shapes[3].step_busy : shapes[3].step_short) * (bits == 4 ? 1.0 : shapes[3].other_bits);
+    const double per_step = (busy ? shapes[3].step_busy : shapes[3].step_short) * (bits == 4 ? 1.0 : shapes[3].other_bits) *
+                            (byte_codes ? shapes[3].bytes : 1.0);
     const double cost = static_cast<double>((tiles + 255) / 256) * (7.5 + steps / 4.0 * per_step);
     if (cost < best_cost) {
       best = 4;
@@ -112,7 +115,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
   g.M = M; g.N = N; g.K = K; g.out = out; g.out_dtype = out_dtype;
   g.out_map = OutMap{out_map, out_map != nullptr && out_dtype == OQ_BF16 ? kWideLoBf16 : -1};
-  int tile = gemm_choose_tile(M, N, K, bits);
+  int tile = choose_tile_with_cost(M, N, K, bits, nullptr, a_mode == A_U8);
   if (a_mode != A_NIBBLE && a_mode != A_U8) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
   g.k_splits = 1;
   const int splits = gemm_choose_splits(M, N, K, bits);
