@@ -294,7 +294,7 @@ def test_packed_linear_tile_kernel(dev, m, n, k, wbits, abits, block, with_bias,
 @pytest.mark.parametrize(("m", "n", "k", "wbits", "abits"), [
     (300, 200, 1024, 4, 6), (130, 96, 256, 4, 8), (257, 384, 1536, 3, 6), (64, 64, 64, 2, 5), (100, 136, 512, 6, 6),
     (90, 72, 384, 8, 8), (515, 520, 1152, 4, 4)])
-@pytest.mark.parametrize("tile", ["0", "1", "3"])
+@pytest.mark.parametrize("tile", ["0", "1", "2", "3", "4"])
 def test_packed_linear_byte_codes_tile_kernel(dev, m, n, k, wbits, abits, tile, library_switch):
     """One activation code per byte (a_bits up to 8) through the all-table tile kernel."""
     library_switch("OQ_GEMM_TILE", tile)
