@@ -204,7 +204,7 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
  * block, the gate and up projections of an MLP): out[i] = oq_packed_linear(codes, ..., packed_w[i],
  * w_bits[i], row_norms[i], w_centroids[i], bias[i], M, N[i], K), bit for bit.  The argument arrays
  * (count entries each, read during the call only) live in host memory and hold device pointers;
- * `bias` may be NULL (no matrix has one) or hold NULL entries.  For at most sixteen tokens, nibble
+ * `bias` may be NULL (no matrix has one) or hold NULL entries.  For at most 32 tokens, nibble
  * codes, 2-, 3- or 4-bit weights and two to four matrices the whole group is ONE launch of the
  * streaming kernel (at decode sizes a launch is mostly fixed cost); any other group runs as
  * `count` launches.  No counterpart in the reference, whose layers each call

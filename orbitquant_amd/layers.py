@@ -344,7 +344,7 @@ class OrbitLinearGroup:
     called together: `q, k, v = OrbitLinearGroup(attn.q, attn.k, attn.v)(x)`.
 
     The whole group is one native call (`oq_quantized_linear_group`): the input is quantized once,
-    and the packed linears of at most sixteen tokens are one launch.  Every output equals the module's
+    and the packed linears of at most 32 tokens are one launch.  Every output equals the module's
     own `forward(x)` bit for bit.  The group holds references to the modules, not copies, and is not
     itself a module: parameters and state dict stay where they are.  The members must share
     `in_features`, rotation, activation width and fused input activation; under `torch.compile`, or

@@ -73,12 +73,19 @@ GROUPS = [
     dict(m=5, k=2048, shapes=[(4096, 4, True), (1000, 3, False)], abits=4),
     # more rows than the rule for one / two rows-per-workgroup steps
     dict(m=2, k=512, shapes=[(5000, 3, False), (4200, 3, False)], abits=4),
+    # 17 to 64 tokens: the single launch with two or four blocks of sixteen token rows per workgroup
+    dict(m=17, k=512, shapes=[(96, 2, False), (40, 2, True), (17, 3, False)], abits=4),
+    dict(m=32, k=4096, shapes=[(1024, 2, False), (256, 2, False), (250, 3, False)], abits=4),
+    dict(m=64, k=2048, shapes=[(4096, 4, True), (1000, 3, False)], abits=4),
+    dict(m=33, k=512, shapes=[(5000, 3, False), (4200, 3, False)], abits=4),
+    dict(m=64, k=384, shapes=[(64, 3, False), (64, 4, False), (64, 2, False), (33, 3, True)], abits=3),
+    dict(m=48, k=1024, shapes=[(9000, 4, True), (8200, 2, False)], abits=4),
     # groups that run as one launch per matrix: mixed K-splits, byte codes, wide weights, many tokens,
     # more than four matrices, a single matrix
     dict(m=1, k=4096, shapes=[(4096, 4, False), (4112, 4, False)], abits=4),
     dict(m=4, k=512, shapes=[(64, 4, False), (48, 3, True)], abits=6),
     dict(m=4, k=512, shapes=[(64, 6, False), (48, 8, True)], abits=4),
-    dict(m=40, k=512, shapes=[(64, 4, False), (48, 3, True)], abits=4),
+    dict(m=70, k=512, shapes=[(64, 4, False), (48, 3, True)], abits=4),
     dict(m=1, k=256, shapes=[(32, 2, False)] * 5, abits=4),
     dict(m=1, k=256, shapes=[(32, 4, True)], abits=4),
 ]
