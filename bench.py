@@ -512,7 +512,9 @@ def build_c5(device, gen):
     return mats
 
 
-def bench_c5(args, device):
+def measure_c5(args, device, brief=False):
+    """The decode stack as the step; returns the JSON line of `--workload c5` (brief: without the C-ABI
+    and kernel-only legs, for the extra key of the default line)."""
     from orbitquant_amd import ops
 
     gen = torch.Generator().manual_seed(5)
@@ -576,6 +578,10 @@ def bench_c5(args, device):
         if graph_dt < dt:
             dt, launch = graph_dt, "hipgraph"
 
+    if brief:
+        return {"ms_per_step": dt * 1e3, "gbs": packed_bytes / dt / 1e9, "frac_of_hbm": packed_bytes / dt / 1e9 / HBM_PEAK_GBS, "M": m,
+                "launch": launch, "packed_bytes_per_step": packed_bytes,
+                "workload": "c5 40-layer decode stack W2/W3/W4 A4: quantize + packed linear of q, k, v (one group), o, up, down per layer"}
     # The same stack driven through the C ABI alone (what a native host does: one oq_quantized_linear
     # call per linear into buffers it owns, no module, no op dispatch, no allocation), to separate
     # the library from the Python around it.  Reported beside `value`, not as `value`.
@@ -634,6 +640,11 @@ def bench_c5(args, device):
         "roofline": dict(small_m_roofline(device, args.kernel_iters, m=m), stack_matmuls_gbs=packed_bytes / per_stack / 1e9,
                          stack_w4_up_avg_launch_us=per_w4 * 1e6, stack_w4_up_gbs=achieved),
     }
+    return out
+
+
+def bench_c5(args, device):
+    out = measure_c5(args, device)
     copy_calibration(device)
     print(json.dumps(out))
 
@@ -719,6 +730,7 @@ def main() -> int:
         out["roofline_small_m"] = small_m_roofline(device, args.kernel_iters)
         out["c3_gemms"] = c3_gemm_lines(device, args.kernel_iters)
         out["float_activations"] = float_activation_lines(device, args.kernel_iters)
+        out["decode_stack"] = measure_c5(args, device, brief=True)
     copy_calibration(device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(spec, layers, x)
