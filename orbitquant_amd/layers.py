@@ -145,7 +145,7 @@ class OrbitLinear(nn.Module):
         self.register_buffer("_nibble_weight_copy", None, persistent=False)
         self.register_buffer("_nibble_weight_centroids", None, persistent=False)
 
-    MANY_TOKENS = 256
+    MANY_TOKENS = 65   # from here on the matmul is the tile kernel (up to 64 tokens: the streaming kernel)
 
     def prepare_many_token_weights(self) -> None:
         """Build the four-bit copy of a 2- or 3-bit index stream now (it is otherwise built by the first
@@ -167,7 +167,8 @@ class OrbitLinear(nn.Module):
         by instruction issue there, not by weight bytes, and extracting 3-bit fields that straddle bytes
         (or four 2-bit fields per byte) costs it 11-22 % against whole nibbles, so it is given the same
         indices at four bits each, with the codebook padded to sixteen entries.  Same operand values,
-        same sums.  Decode-sized calls, which are bound by the bytes, keep reading the stored stream."""
+        same sums.  Measured from 65 tokens (7-17 % there) to several thousand.  Calls of up to 64 tokens
+        take the streaming kernel, which is bound by decode work per byte, and keep reading the stored stream."""
         if (self.weight_bits in (2, 3) and self.nibble_copy_for_many_tokens and tokens >= self.MANY_TOKENS
                 and self.packed_weight_indices.device.type == "cuda"):
             if self._nibble_weight_copy is None and not torch.compiler.is_compiling():

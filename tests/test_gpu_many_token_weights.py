@@ -30,7 +30,7 @@ def make_layer(dev, k, n, wbits, abits, bias=True, seed=0):
 
 @pytest.mark.parametrize("k,n,wbits,abits,m", [
     (1152, 1152, 3, 3, 512), (1024, 600, 2, 4, 300), (3072, 1024, 3, 3, 4608), (512, 200, 3, 6, 257),
-    (1088, 96, 2, 3, 256), (2048, 4096, 3, 4, 1000)])
+    (1088, 96, 2, 3, 256), (2048, 4096, 3, 4, 1000), (4096, 520, 3, 4, 65), (1024, 256, 2, 4, 100)])
 def test_copy_gives_the_outputs_of_the_stored_stream(dev, k, n, wbits, abits, m):
     from orbitquant_amd import ops
 
@@ -58,9 +58,9 @@ def test_copy_follows_the_weights(dev):
     small, many = torch.randn(16, 1024, device=dev, dtype=torch.bfloat16), torch.randn(256, 1024, device=dev, dtype=torch.bfloat16)
     layer(small)
     assert layer._nibble_weight_copy is None                  # decode-sized calls read the stored stream
-    assert layer._matmul_weight(255)[1] == 3 and layer._nibble_weight_copy is None
+    assert layer._matmul_weight(64)[1] == 3 and layer._nibble_weight_copy is None
     first = layer(many)
-    assert layer._nibble_weight_copy is not None and layer._matmul_weight(256)[1] == 4
+    assert layer._nibble_weight_copy is not None and layer._matmul_weight(65)[1] == 4
     assert "_nibble_weight_copy" not in layer.state_dict()
     # other weights loaded into the same module: the copy is dropped and rebuilt from them
     other = make_layer(dev, 1024, 512, 3, 4, seed=9)
