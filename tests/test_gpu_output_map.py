@@ -80,6 +80,21 @@ def test_output_map_equals_function_of_plain_output(dev, m, k, n, wbits, abits, 
     assert torch.equal(linear(c, output_map=table), fn(plain))
 
 
+@pytest.mark.parametrize("m,k,n,splits", [(200, 2048, 256, "2"), (128, 8192, 520, "8"), (48, 2048, 256, None)])
+def test_output_map_behind_shared_k_and_row_blocks(dev, m, k, n, splits, library_switch):
+    """The map after a GEMM that shares K between workgroups (applied by a launch of its own, after the parts
+    are added) and after the streaming kernel at 17 to 64 tokens."""
+    from orbitquant_amd import ops
+
+    if splits is not None:
+        library_switch("OQ_GEMM_WG_SPLIT", splits)
+    c = make_case(dev, m, k, n, 4, 4, torch.bfloat16, seed=m + k + n)
+    table = ops.activation_table(gelu, torch.bfloat16, dev)
+    plain = linear(c)
+    assert torch.isfinite(plain.float()).all()
+    assert torch.equal(linear(c, output_map=table), gelu(plain))
+
+
 def test_packed_linear_mapped_entry_point(dev):
     from orbitquant_amd import _lib, ops
 
