@@ -379,6 +379,40 @@ def test_packed_linear_k_shared_between_workgroups(dev, m, n, k, wbits, abits, s
     check_outputs(fp32, oracle_linear(layer, codes, s, torch.float32), s, layer["r"].float().numpy(), k, "fp32 out")
 
 
+def test_packed_linear_shared_k_is_skipped_under_graph_capture(dev, library_switch):
+    """A captured stream gets the single launch (the buffer of partial tiles may have to grow, which a graph cannot
+    record): the replay returns the bits of the eager single launch."""
+    rng = np.random.default_rng(5)
+    m, n, k = 128, 256, 8192
+    layer = make_layer(rng, n, k, 4, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    library_switch("OQ_GEMM_WG_SPLIT", "1")
+    single = run_packed_linear(dev, layer, codes, s, "nibble")
+    library_switch("OQ_GEMM_WG_SPLIT", "8")
+    split = run_packed_linear(dev, layer, codes, s, "nibble")
+    assert not torch.equal(split, single)          # the eager call does share K here
+    from orbitquant_amd import ops
+    args = (torch.from_numpy(o.pack_nibbles(codes)).to(dev), torch.from_numpy(s).to(dev), torch.from_numpy(layer["ca"]).to(dev),
+            torch.from_numpy(layer["packed"]).to(dev), layer["r"].to(dev), torch.from_numpy(layer["cw"]).to(dev))
+    kw = dict(code_format="nibble", activation_bits=4, weight_bits=4, out_features=n, in_features=k,
+              bias=torch.from_numpy(layer["bias"]).to(torch.bfloat16).to(dev), output_dtype=torch.bfloat16)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.packed_linear(*args, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.packed_linear(*args, **kw)
+    for _ in range(2):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, single)
+
+
 def test_packed_linear_chooses_shared_k_for_short_and_long_problems(dev):
     """The dispatcher's own choice on a short-and-long problem (few tiles, many K-steps) against the oracle."""
     rng = np.random.default_rng(77)
