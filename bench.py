@@ -259,29 +259,86 @@ def _code_format(layer, x):
     return "u8" if (tokens > 16 and k % 64 == 0) or k % 128 == 0 else None
 
 
+class RawLinear:
+    """One OrbitLinear as bare C-ABI calls into buffers allocated once: what a native host does.
+
+    The Python wrappers in orbitquant_amd/ops.py check every operand and allocate the outputs of every
+    call; at the c2 shapes that is more host time per call than the kernels take on the device, and a
+    loop of such calls measures the host.  These closures call the library the way bench.py's kernel
+    timings need it: same entry points, same operands, nothing else."""
+
+    def __init__(self, layer, x, with_output_map=True):
+        from orbitquant_amd import _lib, ops
+
+        self.lib = _lib.load()
+        self.layer, self.x = layer, x
+        k, n = layer.in_features, layer.out_features
+        m = x.numel() // k
+        self.m, self.k, self.n = m, k, n
+        dev = x.device
+        self.fmt = _code_format(layer, x)
+        if self.fmt is None:
+            raise ValueError("this layer's forward passes values, not codes")
+        width = k // 2 if self.fmt == "nibble" else k
+        self.codes = torch.empty((m, width), dtype=torch.uint8, device=dev)
+        self.norms = torch.empty(m, dtype=torch.float32, device=dev)
+        self.out = torch.empty((m, n), dtype=x.dtype, device=dev)
+        dt = ops._DTYPES[x.dtype]
+        fmt = {"u8": ops.OQ_CODES_U8, "nibble": ops.OQ_CODES_NIBBLE}[self.fmt]
+        packed, w_bits, w_cents = layer._matmul_weight(m)   # what the layer's forward reads at this token count
+        self.keep = (packed, w_cents)
+        levels = layer._activation_codebook_boundaries.numel() + 1
+        imap = layer._input_activation_table
+        omap = layer._output_activation_table if with_output_map else None
+        plan = layer._rotation_plan
+        rot = (layer._rotation_permutation.data_ptr(), layer._rotation_signs.data_ptr(),
+               layer._activation_codebook_boundaries.data_ptr(), layer._activation_codebook_centroids.data_ptr())
+        consts = (int(layer.rotation.block_size), float(layer.activation_eps), float(layer.rotation.normalization))
+        q_tail = (self.codes.data_ptr(), fmt, None, ops.OQ_VALUES_NONE, self.norms.data_ptr())
+        if imap is None:
+            self._quantize = (self.lib.oq_rotate_quantize,
+                              (x.data_ptr(), dt, m, k, *rot, levels, *consts, ops._ptr(plan), *q_tail))
+        else:
+            self._quantize = (self.lib.oq_rotate_quantize_mapped,
+                              (x.data_ptr(), dt, imap.data_ptr(), m, k, *rot, levels, *consts, *q_tail))
+        bias = layer.bias
+        g_args = (self.codes.data_ptr(), fmt, self.norms.data_ptr(), layer._activation_codebook_centroids.data_ptr(),
+                  int(layer.activation_bits), packed.data_ptr(), int(w_bits), layer.row_norms.data_ptr(), w_cents.data_ptr(),
+                  ops._ptr(bias), ops._dt(bias) if bias is not None else ops.OQ_F32, m, n, k, self.out.data_ptr(), dt)
+        self._gemm = ((self.lib.oq_packed_linear, g_args) if omap is None else
+                      (self.lib.oq_packed_linear_mapped, (*g_args, omap.data_ptr())))
+        self._linear = (self.lib.oq_quantized_linear,
+                        (x.data_ptr(), dt, ops._ptr(imap), m, k, *rot, int(layer.activation_bits), *consts, ops._ptr(plan),
+                         packed.data_ptr(), int(w_bits), layer.row_norms.data_ptr(), w_cents.data_ptr(), ops._ptr(bias),
+                         ops._dt(bias) if bias is not None else ops.OQ_F32, n, self.codes.data_ptr(), self.norms.data_ptr(),
+                         self.out.data_ptr(), dt, ops._ptr(omap)))
+
+    def _call(self, what):
+        fn, args = what   # (the stream is looked up per call: under graph capture it is the capturing stream)
+        if fn(*args, torch.cuda.current_stream().cuda_stream) != 0:
+            raise RuntimeError(self.lib.oq_last_error().decode())
+
+    def quantize(self):
+        self._call(self._quantize)
+
+    def gemm(self):
+        self._call(self._gemm)
+
+    def linear(self):
+        self._call(self._linear)
+        return self.out
+
+
 def gemm_only_closure(layer, x, with_output_map=True):
     """The matmul launch of `layer` alone, on pre-computed activation codes (with the layer's
     fused output activation, as it runs in the step, unless `with_output_map` is False)."""
     from orbitquant_amd import ops
 
     k = layer.in_features
-    fmt = _code_format(layer, x)
-    if fmt is not None:
-        codes, _, norms = ops.rotate_quantize(
-            x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
-            block_size=layer.rotation.block_size, eps=layer.activation_eps,
-            inv_sqrt_block=layer.rotation.normalization, code_format=fmt,
-            input_map=layer._input_activation_table, plan=layer._rotation_plan)
-        bias = layer.bias
-        packed, weight_bits, weight_centroids = layer._matmul_weight(x.numel() // k)  # what the layer's forward reads
-
-        def fn():
-            return ops.packed_linear(
-                codes, norms, layer._activation_codebook_centroids, packed, layer.row_norms,
-                weight_centroids, code_format=fmt, activation_bits=layer.activation_bits,
-                weight_bits=weight_bits, out_features=layer.out_features, in_features=k, bias=bias,
-                output_dtype=x.dtype, output_map=layer._output_activation_table if with_output_map else None)
-        return fn
+    if _code_format(layer, x) is not None:
+        raw = RawLinear(layer, x, with_output_map)
+        raw.quantize()
+        return raw.gemm
     _, unit, norms = ops.rotate_quantize(
         x, layer._rotation_permutation, layer._rotation_signs, layer._activation_codebook_boundaries,
         block_size=layer.rotation.block_size, eps=layer.activation_eps,
@@ -301,7 +358,9 @@ def quantize_only_closure(layer, x):
     from orbitquant_amd import ops
 
     fmt = _code_format(layer, x)
-    vals = None if fmt else "unit_bf16"
+    if fmt is not None:
+        return RawLinear(layer, x).quantize
+    vals = "unit_bf16"
 
     def fn():
         return ops.rotate_quantize(
@@ -310,6 +369,28 @@ def quantize_only_closure(layer, x):
             inv_sqrt_block=layer.rotation.normalization, centroids=layer._activation_codebook_centroids,
             code_format=fmt, values=vals, input_map=layer._input_activation_table, plan=layer._rotation_plan)
     return fn
+
+
+def abi_step_closure(layers, x):
+    """The whole step as bare C-ABI calls (one oq_quantized_linear per layer into buffers allocated once),
+    or None when a layer of the step has no such form (a separate activation kernel, value activations)."""
+    if any(act == "gelu" and not activation_is_fused(layers, i) for i, (_l, act) in enumerate(layers)):
+        return None
+    raws, h = [], x
+    for layer, act in layers:
+        if _code_format(layer, h) is None:
+            return None
+        raw = RawLinear(layer, h)
+        raws.append(raw)
+        h = raw.out
+        if act == "slice3072":
+            return None
+
+    def step():
+        for raw in raws:
+            raw.linear()
+        return raws[-1].out
+    return step
 
 
 # ----------------------------------------------------------------- CPU baseline
@@ -430,10 +511,25 @@ def small_m_roofline(device, iters, m=1, copies=16):
     row_norms = torch.full((n,), 1.28).to(torch.bfloat16).to(device)
     mats = [torch.randint(0, 256, (n * k * bits // 8,), generator=gen, dtype=torch.uint8).to(device) for _ in range(copies)]
 
+    # bare C-ABI calls into one output buffer (the Python wrapper's checks and allocation take longer
+    # than this kernel runs)
+    from orbitquant_amd import _lib
+    lib = _lib.load()
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    calls = [(codes.data_ptr(), ops.OQ_CODES_NIBBLE, norms.data_ptr(), cents.data_ptr(), 4, w.data_ptr(), bits,
+              row_norms.data_ptr(), cents.data_ptr(), None, ops.OQ_F32, m, n, k, out.data_ptr(), ops.OQ_BF16)
+             for w in mats]
+    want = ops.packed_linear(codes, norms, cents, mats[-1], row_norms, cents, code_format="nibble", activation_bits=4,
+                             weight_bits=bits, out_features=n, in_features=k, output_dtype=torch.bfloat16)
+
     def fn():
-        for w in mats:
-            ops.packed_linear(codes, norms, cents, w, row_norms, cents, code_format="nibble", activation_bits=4,
-                              weight_bits=bits, out_features=n, in_features=k, output_dtype=torch.bfloat16)
+        stream = torch.cuda.current_stream().cuda_stream   # (under graph capture: the capturing stream)
+        for c in calls:
+            if lib.oq_packed_linear(*c, stream) != 0:
+                raise RuntimeError(lib.oq_last_error().decode())
+    fn()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want), "bare call differs from the wrapper's"
     per_launch = time_kernel(fn, max(3, iters // 5)) / copies
     nbytes = mats[0].numel() + 2 * n
     achieved = nbytes / per_launch / 1e9
@@ -676,10 +772,23 @@ def main() -> int:
     eager_dt = time_steps(lambda: run_step(layers, x), args.steps, args.warmup)
     dt, launch, graph_dt = eager_dt, "eager", None
     captured = None if args.no_graph else capture_step(lambda: run_step(layers, x))
-    if captured is not None:   # both ways of launching are timed; `value` is the faster, `config.launch` says which
+    if captured is not None:   # every way of launching is timed; `value` is the fastest, `config.launch` says which
         graph_dt = time_steps(captured[0], args.steps, args.warmup)
         if graph_dt < dt:
             dt, launch = graph_dt, "hipgraph"
+    # the same step driven through the C ABI alone: one oq_quantized_linear call per layer into buffers
+    # allocated once (no module, no op dispatch, no allocation per call); same kernels, same outputs
+    abi_dt = None
+    abi = abi_step_closure(layers, x)
+    if abi is not None:
+        want = run_step(layers, x)
+        got = abi()
+        torch.cuda.synchronize()
+        if not torch.equal(got, want):
+            raise AssertionError("the C-ABI step differs from the module step")
+        abi_dt = time_steps(abi, args.steps, args.warmup)
+        if abi_dt < dt:
+            dt, launch = abi_dt, "c_abi"
 
     # dominant kernel alone: the packed GEMM of the first layer, and every other piece for the record
     pieces = {}
@@ -709,6 +818,7 @@ def main() -> int:
         "config": {"workload": spec["name"], "M": spec["M"], "input_dtype": str(spec["dtype"]).replace("torch.", ""),
                    "flop_per_step": flops, "launch": launch, "eager_ms_per_step": eager_dt * 1e3,
                    "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
+                   "c_abi_ms_per_step": None if abi_dt is None else abi_dt * 1e3,
                    "preroll_s": PREROLL_SECONDS,
                    "activation": ("gelu as a 65536-entry table of torch's own results, looked up in the producing "
                                   "matmul's epilogue" if any(l._output_activation_table is not None for l, _ in layers)

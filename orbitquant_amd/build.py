@@ -5,6 +5,13 @@
 hipcc cross-compiles for gfx950 without a GPU.  The rotate+quantize kernel is
 built without FMA contraction (its results must match the CPU statement of the
 algorithm bit for bit); packed fp32 VALU instructions are disabled everywhere.
+
+    python -m orbitquant_amd.build --variant stamps --flags=-DOQ_GEMM_STAMPS --only packed_gemm.hip
+
+builds `liborbitquant_hip_stamps.so` beside the library: the listed sources compiled with the
+extra flags, every other object taken from the last full build.  `ORBITQUANT_HIP_LIB=<path>`
+makes the package load it.  (-DOQ_GEMM_STAMPS: the tile GEMM records the clock at its phase
+boundaries, see `bench.py --gemm-phases`.)
 """
 
 from __future__ import annotations
@@ -52,9 +59,9 @@ SOURCES = {
 INCREMENTAL = False
 
 
-def _compile(item) -> Path:
+def _compile(item, obj_dir: Path = None) -> Path:
     name, extra = item
-    obj = OBJ_DIR / (name + ".o")
+    obj = (obj_dir or OBJ_DIR) / (name + ".o")
     if INCREMENTAL and obj.exists():
         newest = max(p.stat().st_mtime for p in list(CSRC.glob("*.h")) + [CSRC / name, PKG.parent / "include/orbitquant_hip.h"])
         if obj.stat().st_mtime > newest:
@@ -83,7 +90,34 @@ def build(verbose: bool = True) -> Path:
     return LIB
 
 
+def build_variant(variant: str, flags: list, only: list) -> Path:
+    """The library with `only` recompiled under `flags`; the other objects come from the full build."""
+    obj_dir = PKG / f"build_{variant}"
+    obj_dir.mkdir(exist_ok=True)
+    missing = [n for n in SOURCES if n not in only and not (OBJ_DIR / (n + ".o")).exists()]
+    if missing:
+        raise SystemExit(f"run the full build first: no object for {missing}")
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        changed = dict(zip(only, pool.map(lambda n: _compile((n, SOURCES[n] + flags), obj_dir), only)))
+    objects = [str(changed.get(n, OBJ_DIR / (n + ".o"))) for n in SOURCES]
+    lib = PKG / f"liborbitquant_hip_{variant}.so"
+    subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib)] + objects, check=True)
+    print("built", lib)
+    return lib
+
+
 if __name__ == "__main__":
-    INCREMENTAL = "--incremental" in sys.argv
-    build()
+    import argparse
+
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--incremental", action="store_true")
+    ap.add_argument("--variant", default=None)
+    ap.add_argument("--flags", default="")
+    ap.add_argument("--only", default="")
+    opts = ap.parse_args()
+    INCREMENTAL = opts.incremental
+    if opts.variant:
+        build_variant(opts.variant, opts.flags.split(), [n for n in opts.only.split(",") if n])
+    else:
+        build()
     sys.exit(0)

@@ -52,7 +52,7 @@ bool reserve_dynamic_lds(const void *kernel, size_t bytes) {
 namespace {
 const char *const kEnvNames[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", "OQ_RQ_ONE_GROUP", "OQ_GEMV_CFG", "OQ_RQ_WAVES",
                                           "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE",
-                                          "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT", "OQ_FLOAT_GEMM_MIN_M"};
+                                          "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT", "OQ_FLOAT_GEMM_MIN_M", "OQ_GEMM_STAMPS"};
 const char *env_values[ENV_COUNT];
 void env_load() {
   static std::once_flag once;

@@ -22,7 +22,7 @@ const char *debug_env(int which);
 // (oq_quantized_linear_static): stream_workspace() then hands out nothing, and the dispatchers take
 // the paths that need no buffer.
 bool allocation_forbidden();
-enum DebugEnv { ENV_GEMM_TILE = 0, ENV_NO_TOKEN_LINEAR, ENV_RQ_ONE_GROUP, ENV_GEMV_CFG, ENV_RQ_WAVES, ENV_RQ_FAST_MIN_M, ENV_NO_GEMV_GROUP, ENV_GEMV_GROUP_R, ENV_GEMV_NO_ASTAGE, ENV_GEMV_MAX_M, ENV_GEMM_WG_SPLIT, ENV_FLOAT_GEMM_MIN_M, ENV_COUNT };
+enum DebugEnv { ENV_GEMM_TILE = 0, ENV_NO_TOKEN_LINEAR, ENV_RQ_ONE_GROUP, ENV_GEMV_CFG, ENV_RQ_WAVES, ENV_RQ_FAST_MIN_M, ENV_NO_GEMV_GROUP, ENV_GEMV_GROUP_R, ENV_GEMV_NO_ASTAGE, ENV_GEMV_MAX_M, ENV_GEMM_WG_SPLIT, ENV_FLOAT_GEMM_MIN_M, ENV_GEMM_STAMPS, ENV_COUNT };
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -256,17 +256,62 @@ __device__ __forceinline__ void write_row_tables(uint32_t *lds, uint32_t my_w, u
   }
 }
 
-// dword of weight-table row e
-template <int BITS>
-__device__ __forceinline__ uint32_t w_table_entry(const float *cents, int e) {
-  constexpr int levels = 1 << BITS;
-  if constexpr (BITS <= 4) {
-    if (e >= levels * levels) return 0u;
-    return pack16(cents[e & (levels - 1)], cents[e >> BITS], false);
-  } else {
-    if (e >= levels) return 0u;
-    const float v = cents[e];
-    return pack16(v, v, false);
+// The same block without a lane exchange, for pair tables (weights of 2, 3 or 4 bits; activation codes two
+// per byte or no activation table at all).  Lane l of wavefront w writes 16-byte chunk l % 16 of rows
+// 64 w + 4 i + l / 16, i = 0..15: a weight copy (chunks 0..7) or an activation copy.  The entry of row e is
+// (c[e mod L], c[(e >> bits) mod L]), and for the rows of one lane  e mod L = (4 i + l / 16) mod L  takes four
+// values while  e >> bits  takes at most eight, the same for every lane of the wavefront: a lane loads those
+// centroids itself (request_pair_seed, with the kernel's other first loads) and every entry is one conversion
+// instruction.  (The exchange-based build is a chain of sixteen LDS round trips per wavefront: 0.8 us of a
+// 25 us launch.)  Weight rows past L * L are never indexed and hold arbitrary entries.
+template <int BITS, bool HAS_A>
+__device__ __forceinline__ void request_pair_seed(float (&lo_w)[4], float (&hi_w)[8], float (&lo_a)[4], float (&hi_a)[4],
+                                                  const float *__restrict__ w_cents,
+                                                  const float *__restrict__ act_cents, int a_levels) {
+  static_assert(BITS >= 2 && BITS <= 4, "pair tables");
+  constexpr int L = 1 << BITS;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lo_w[j] = w_cents[(4 * j + g) & (L - 1)];
+  // e >> bits for rows 64 w + 4 i + g:  4 w + i / 4 (16 levels),  i / 2 (8 levels, rows below 64),  i (4 levels, rows below 16)
+#pragma unroll
+  for (int t = 0; t < 8; ++t) hi_w[t] = t < (BITS == 3 ? 8 : 4) ? w_cents[BITS == 4 ? ((4 * wave + t) & 15) : t] : 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    lo_a[j] = HAS_A ? act_cents[min(4 * j + g, a_levels - 1)] : 0.0f;
+    hi_a[j] = HAS_A ? act_cents[min(4 * wave + j, a_levels - 1)] : 0.0f;
+  }
+}
+
+template <int BITS, bool HAS_A>
+__device__ __forceinline__ void write_pair_tables(uint32_t *lds, const float (&lo_w)[4], const float (&hi_w)[8],
+                                                  const float (&lo_a_raw)[4], const float (&hi_a_raw)[4], int a_levels) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4;
+  const bool is_a = (lane & 8) != 0;
+  float lo_a[4], hi_a[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {  // codes past the table read zero
+    lo_a[j] = (HAS_A && 4 * j + g < a_levels) ? lo_a_raw[j] : 0.0f;
+    hi_a[j] = (HAS_A && 4 * wave + j < a_levels) ? hi_a_raw[j] : 0.0f;
+  }
+  // a lane writes either weight or activation copies: choose the operands once
+  float lo[4], hi[16];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lo[j] = is_a ? lo_a[j] : lo_w[j];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int slot = BITS == 4 ? (i >> 2) : BITS == 3 ? (i >> 1) : (i & 3);
+    if (BITS == 4 && (i & 3)) hi[i] = hi[i & ~3];
+    else hi[i] = is_a ? hi_a[i >> 2] : hi_w[slot];
+  }
+  unsigned char *row0 = reinterpret_cast<unsigned char *>(lds) + (64 * wave + g) * 256 + (lane & 15) * 16;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const f32x2_t pair = {lo[i & 3], hi[i]};
+    const uint32_t d = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+    *reinterpret_cast<uint4 *>(row0 + i * 1024) = make_uint4(d, d, d, d);
   }
 }
 

@@ -118,6 +118,7 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   int tile = choose_tile_with_cost(M, N, K, bits, nullptr, a_mode == A_U8);
   if (a_mode != A_NIBBLE && a_mode != A_U8) return fail(OQ_ERR_INVALID, "packed_gemm: a_mode %d", a_mode);
   g.k_splits = 1;
+  if (const char *where = debug_env(ENV_GEMM_STAMPS)) g.stamps = reinterpret_cast<uint64_t *>(strtoull(where, nullptr, 0));  // builds with -DOQ_GEMM_STAMPS: a device buffer for the kernel's phase stamps
   const int splits = gemm_choose_splits(M, N, K, bits);
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (splits > 1 && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {

@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
   const int64_t m0 = static_cast<int64_t>(pid_m) * TM, n0 = static_cast<int64_t>(pid_n) * TN;
   const int wm = (wave >> 1) * (FM * 32), wn = (wave & 1) * (FN * 32);
 
-  EpiFactors<FM> epi;
-  gemm_epilogue_prefetch<FM>(epi, m0, n0, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+  EpiRaw<FM> epi_raw;
+  gemm_epilogue_request<FM>(epi_raw, m0, n0, wm, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.w_cents);
 
   // ---- A loader: chunk c = tid + 256*i -> row c/8, 16-byte chunk c%8 of the row's 128-byte slab
   const int64_t a_row_bytes = g.K * 2, w_row_bytes = g.K * BITS / 8;
@@ -181,6 +181,8 @@ __global__ __launch_bounds__(256) void packed_gemm_av_kernel(AvArgs g) {
   }
 
   __syncthreads();  // tables and staging buffers are dead: LDS is reused by the epilogue
+  EpiFactors<FM> epi;
+  gemm_epilogue_factors<FM>(epi, epi_raw, TN, tid, g.row_scale != nullptr, g.bias != nullptr, g.bias_dtype);
   gemm_epilogue<FM, FN>(acc, m0, n0, wm, wn, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, g.out,
                         g.out_dtype, reinterpret_cast<unsigned char *>(lds), g.out_map);
 }

@@ -72,6 +72,10 @@ struct GemmArgs {
   // adds them up and applies the epilogue.
   int k_splits;
   float *partials;
+  int window_ahead;          // the launch has kWideBytes of dynamic LDS for the output map's window (set by launch_cfg)
+  // Builds with -DOQ_GEMM_STAMPS only: every wavefront writes the shader-clock and real-time counter
+  // values it read at its phase boundaries to stamps[(workgroup * 4 + wavefront) * 16 ...] (NULL: none).
+  uint64_t *stamps;
 };
 
 void *stream_workspace(size_t bytes, hipStream_t stream);  // packed_gemm_tiled.hip
@@ -95,20 +99,66 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, grp = lane >> 5;
+#ifdef OQ_GEMM_STAMPS
+  uint64_t stamp[8], stamp_extra[4] = {0, 0, 0, 0};
+  stamp[0] = __builtin_amdgcn_s_memtime();
+  stamp[6] = __builtin_amdgcn_s_memrealtime();
+#define OQ_STAMP(i) stamp[i] = __builtin_amdgcn_s_memtime()
+#else
+#define OQ_STAMP(i)
+#endif
 
-  // Loads of one wavefront return in order, so the centroid values this thread needs for its
-  // table row are requested first, then the packed operands of the first K-steps; the tables
-  // are written while the packed data is still in flight.
-  const uint32_t my_w = w_table_entry<BITS>(g.w_cents, tid);
-  uint32_t my_a;
-  if constexpr (AM == A_TILED || AM == A_STAGED) {
-    my_a = 0u;                     // no activation table
-  } else if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
-    const int c0 = tid & 15, c1 = tid >> 4;
-    my_a = pack16(c0 < g.a_levels ? g.act_cents[c0] : 0.0f, c1 < g.a_levels ? g.act_cents[c1] : 0.0f, false);
-  } else {                         // row = one code, its value in both halves of the dword
-    const float v = tid < g.a_levels ? g.act_cents[tid] : 0.0f;
-    my_a = pack16(v, v, false);
+  // Loads of one wavefront return in order, and the compiler waits for a load where its value is
+  // first touched.  So everything the prologue needs from memory is REQUESTED here, branch-free
+  // (indices clamped into the tables, nothing loaded on one side of a branch only), in the order
+  // centroids, epilogue factors, packed operands of the first K-steps, and nothing is looked at
+  // before the last of these requests has been issued: the tables are then written while the
+  // packed data is still in flight.  (Converting a centroid where it was loaded put one memory
+  // round trip per table operand in front of the first operand load of every workgroup.)
+  constexpr bool kPairTables = BITS <= 4 && AM != A_U8;  // built without a lane exchange (packed_decode.h)
+  constexpr bool kHasATable = AM == A_NIBBLE || AM == A_U8;
+  constexpr int kWLevels = 1 << BITS;
+  float seed_lo_w[4], seed_hi_w[8], seed_lo_a[4], seed_hi_a[4];
+  float w_c0 = 0.0f, w_c1 = 0.0f, a_c0 = 0.0f, a_c1 = 0.0f;
+  bool w_row_used = false, a_ok0 = false, a_ok1 = false;
+  if constexpr (kPairTables) {
+    request_pair_seed<BITS, kHasATable>(seed_lo_w, seed_hi_w, seed_lo_a, seed_hi_a, g.w_cents, g.act_cents, g.a_levels);
+  } else {  // thread t holds the two dwords of row t, handed round by write_row_tables
+    const int w_i0 = tid & (kWLevels - 1), w_i1 = BITS <= 4 ? (tid >> BITS) & (kWLevels - 1) : w_i0;
+    w_c0 = g.w_cents[w_i0];
+    w_c1 = g.w_cents[w_i1];
+    w_row_used = BITS <= 4 ? tid < kWLevels * kWLevels : tid < kWLevels;
+    if constexpr (AM == A_NIBBLE) {  // row = a byte of the stream = two codes
+      const int c0 = tid & 15, c1 = tid >> 4;
+      a_ok0 = c0 < g.a_levels;
+      a_ok1 = c1 < g.a_levels;
+      a_c0 = g.act_cents[min(c0, g.a_levels - 1)];
+      a_c1 = g.act_cents[min(c1, g.a_levels - 1)];
+    } else if constexpr (AM == A_U8) {  // row = one code, its value in both halves of the dword
+      a_ok0 = a_ok1 = tid < g.a_levels;
+      a_c0 = a_c1 = g.act_cents[min(tid, g.a_levels - 1)];
+    }
+  }
+  // The window of an output map (an activation function as a table, gemm_epilogue.h) is requested with
+  // the rest and parked in LDS behind the tables (16 KB of dynamic LDS, which mapped launches ask for),
+  // so that the epilogue finds it there instead of starting with a memory round trip of its own.
+  extern __shared__ __attribute__((aligned(16))) unsigned char map_window[];
+  const bool window_ahead = g.window_ahead != 0;  // uniform
+  // (requested without a branch - a launch without a map reads the first bytes of the weights - and held as
+  // native vectors: an array of the struct type would be pinned in scratch memory)
+  lds_u32x4 window_piece0, window_piece1, window_piece2, window_piece3;
+  {
+    constexpr int kChunksPerSign = (2 << kWideLog2) / 16;
+    const unsigned char *window_from = window_ahead ? reinterpret_cast<const unsigned char *>(g.out_map.table + g.out_map.lo)
+                                                    : reinterpret_cast<const unsigned char *>(g.w);
+    auto piece = [&](int v) {
+      const int i = tid + 256 * v, sign = i / kChunksPerSign, j = i % kChunksPerSign;
+      return *reinterpret_cast<const lds_u32x4 *>(window_from + (window_ahead ? (sign << 16) + 16 * j : 0));
+    };
+    window_piece0 = piece(0);
+    window_piece1 = piece(1);
+    window_piece2 = piece(2);
+    window_piece3 = piece(3);
   }
 
   constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
@@ -116,6 +166,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // contiguous chunks, then walk groups of 4 tile-rows column by column
   int bid = blockIdx.x;
   const int total = g.tiles_m * g.tiles_n;
+#ifdef OQ_GEMM_STAMPS
+  __asm__ volatile("" ::"s"(total));
+  stamp_extra[0] = __builtin_amdgcn_s_memtime();  // kernel arguments have arrived
+#endif
   if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
   constexpr int GROUP_M = 4;
   const int width = GROUP_M * g.tiles_n;
@@ -131,8 +185,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int64_t m_base = static_cast<int64_t>(pid_m) * TM + wm;
   const int64_t n_base = static_cast<int64_t>(pid_n) * TN + wn;
 
-  EpiFactors<FM> epi;
-  gemm_epilogue_prefetch<FM>(epi, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, TN, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype);
+  EpiRaw<FM> epi_raw;
+  gemm_epilogue_request<FM>(epi_raw, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.w_cents);
 
   constexpr int kAStep = AM == A_NIBBLE ? 32 : AM == A_U8 ? 64 : AM == A_TILED ? 4096 : 128;  // bytes from one K-step of 64 to the next in a lane's activation stream
   constexpr int kAVec = AM == A_NIBBLE ? 1 : AM == A_U8 ? 2 : 4;        // 16-byte loads per lane per K-step
@@ -201,7 +255,28 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   fetch(std::integral_constant<int, 0>{}, 0);
   if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
 
-  write_row_tables(lds, my_w, my_a);
+  __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a value may be scheduled above the requests
+  // (first use of the requested values: every request above has been issued)
+#ifdef OQ_GEMM_STAMPS
+  stamp_extra[1] = __builtin_amdgcn_s_memtime();  // every request issued
+  if constexpr (kPairTables) __asm__ volatile("" ::"v"(seed_lo_w[0]), "v"(seed_hi_w[0]), "v"(seed_lo_a[3]), "v"(seed_hi_a[3]));
+  else __asm__ volatile("" ::"v"(w_c0), "v"(w_c1), "v"(a_c0), "v"(a_c1));
+  stamp_extra[2] = __builtin_amdgcn_s_memtime();  // centroids have arrived
+#endif
+  if constexpr (kPairTables) {
+    write_pair_tables<BITS, kHasATable>(lds, seed_lo_w, seed_hi_w, seed_lo_a, seed_hi_a, g.a_levels);
+  } else {
+    const uint32_t my_w = w_row_used ? pack16(w_c0, w_c1, false) : 0u;
+    const uint32_t my_a = pack16(a_ok0 ? a_c0 : 0.0f, a_ok1 ? a_c1 : 0.0f, false);
+    write_row_tables(lds, my_w, my_a);
+  }
+  if (window_ahead) {
+    lds_u32x4 *dst = reinterpret_cast<lds_u32x4 *>(map_window) + tid;
+    dst[0] = window_piece0;
+    dst[256] = window_piece1;
+    dst[512] = window_piece2;
+    dst[768] = window_piece3;
+  }
 
   f32x16 acc[FM][FN];
 #pragma unroll
@@ -210,6 +285,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  OQ_STAMP(1);  // tables written, first operands requested
   __syncthreads();
 
   // ---- main loop: software pipeline over "phases" (one MFMA k-slice of 16) -------
@@ -317,8 +393,21 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
       if (with_fetch && m < FM + FN) fetch_one(fetch_buf, m, fetch_ks);
       const uint4 bw = make_uint4(ob[set ^ 1][j][0], ob[set ^ 1][j][1], ob[set ^ 1][j][2], ob[set ^ 1][j][3]);
       // weights first: the accumulator tile is the transposed output tile
+#ifdef OQ_GEMM_I8_TIMING
+      // Timing experiment only (the results are meaningless): what the loop would cost with the int8 matrix
+      // instruction - half as many matrix instructions, each over twice the K, fed by the same number of lookups.
+      if constexpr ((decltype(mul_q)::value & 1) == 0) {
+        typedef int i32x16_t __attribute__((ext_vector_type(16)));
+        typedef int i32x4_t __attribute__((ext_vector_type(4)));
+        acc[i][j] = __builtin_bit_cast(f32x16, __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            __builtin_bit_cast(i32x4_t, bw), __builtin_bit_cast(i32x4_t, av), __builtin_bit_cast(i32x16_t, acc[i][j]), 0, 0, 0));
+      } else {
+        __asm__ volatile("" ::"v"(bw.x), "v"(bw.y), "v"(bw.z), "v"(bw.w), "v"(av.x), "v"(av.y), "v"(av.z), "v"(av.w));  // the operands stay looked up
+      }
+#else
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, av),
                                                           acc[i][j], 0, 0, 0);
+#endif
 #pragma unroll
       for (int t = lo; t < hi; ++t) lookup_read(buf, q, set, t, addr[m & 1][t - lo]);
       if (m + 1 < kGroups) {
@@ -345,6 +434,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #pragma unroll
   for (int t = 0; t < kLookups; ++t)
     lookup_read(std::integral_constant<int, 0>{}, 0, 0, t, lookup_address(std::integral_constant<int, 0>{}, 0, t));
+  OQ_STAMP(2);  // first operands looked up: the loop starts
   int ks = 0;
   for (; ks + NBUF <= steps; ks += NBUF) {
     step(std::integral_constant<int, 0>{}, ks);
@@ -356,7 +446,11 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     if (NBUF == 3 && ks + 1 < steps) step(std::integral_constant<int, 1>{}, ks + 1);
   }
 
+  OQ_STAMP(3);  // loop done
   __syncthreads();  // every wavefront is done with the lookup tables: LDS is reused from here on
+  OQ_STAMP(4);
+  EpiFactors<FM> epi;
+  gemm_epilogue_factors<FM>(epi, epi_raw, TN, tid, g.row_scale != nullptr, g.bias != nullptr, g.bias_dtype);
   if constexpr (KSPLIT == 1) {
     void *out = g.out;
     int out_dtype = g.out_dtype;
@@ -372,7 +466,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     }
     gemm_epilogue<FM, FN>(acc, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, wn, TN, tid, g.M, g.N,
                           g.row_scale, g.row_norms, g.bias, g.bias_dtype, epi, out, out_dtype,
-                          reinterpret_cast<unsigned char *>(lds), out_map);
+                          reinterpret_cast<unsigned char *>(lds), out_map, 64 * FM,
+                          window_ahead ? reinterpret_cast<const uint16_t *>(map_window) : nullptr);
   } else {
     // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
     // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
@@ -432,8 +527,29 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
 #undef OQ_KSPLIT_ROUND
     gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * wave, 0, TN, tid, g.M,
                          g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
-                         reinterpret_cast<unsigned char *>(lds), g.out_map, TM);
+                         reinterpret_cast<unsigned char *>(lds), g.out_map, TM,
+                         window_ahead ? reinterpret_cast<const uint16_t *>(map_window) : nullptr);
   }
+#ifdef OQ_GEMM_STAMPS
+  OQ_STAMP(5);  // epilogue issued
+  __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  stamp[7] = __builtin_amdgcn_s_memrealtime();
+  const uint64_t done = __builtin_amdgcn_s_memtime();
+  if (g.stamps != nullptr && lane == 0) {
+    uint64_t *dst = g.stamps + (static_cast<int64_t>(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave) * 16;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = stamp[i];
+    dst[8] = done;
+    uint32_t hw;
+    __asm__ volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    uint32_t xcc;
+    __asm__ volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    dst[9] = (static_cast<uint64_t>(xcc) << 32) | hw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[10 + i] = stamp_extra[i];
+  }
+#endif
+#undef OQ_STAMP
 }
 
 template <int AM, int BITS, int FM, int FN, int KSPLIT = 1>
@@ -446,7 +562,10 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   auto kern = packed_gemm_kernel<AM, BITS, FM, FN, KSPLIT>;
   const unsigned splits = (KSPLIT == 1 && (AM == A_NIBBLE || AM == A_U8) && g.k_splits > 1) ? static_cast<unsigned>(g.k_splits) : 1u;
   if (splits == 1) g.k_splits = 1;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), 0, stream, g);
+  // a mapped launch parks the map's window in LDS ahead of its main loop (not for partial tiles: they are not mapped)
+  g.window_ahead = (g.out_map.table != nullptr && g.out_map.lo >= 0 && g.out_dtype == OQ_BF16 && splits == 1 &&
+                    reserve_dynamic_lds(reinterpret_cast<const void *>(kern), kWideBytes)) ? 1 : 0;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), g.window_ahead ? kWideBytes : 0, stream, g);
   return check_launch("packed_gemm");
 }
 
