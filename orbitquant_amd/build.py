@@ -33,6 +33,8 @@ COMMON = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-fno-gpu-flush-denormals-to-zero", "-Wno-unused-command-line-argument",
 ]
+# kernels whose leading scalar arguments are to arrive in scalar registers (see packed_gemm_kernel.h)
+PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
 SOURCES = {
     "capi.hip": [],
     "rotate_quantize.hip": ["-ffp-contract=off"],
@@ -40,13 +42,13 @@ SOURCES = {
     "packed_generic.hip": [],
     "adaln_int4.hip": [],
     "pack_utils.hip": [],
-    "packed_gemm.hip": [],
-    "packed_gemm_bytes.hip": [],
-    "packed_gemm_tiled.hip": [],
-    "packed_gemm_staged.hip": [],
+    "packed_gemm.hip": PRELOAD,
+    "packed_gemm_bytes.hip": PRELOAD,
+    "packed_gemm_tiled.hip": PRELOAD,
+    "packed_gemm_staged.hip": PRELOAD,
     "packed_gemm_splitk.hip": [],
     "packed_gemm_av.hip": [],
-    "packed_gemv.hip": [],
+    "packed_gemv.hip": PRELOAD,
     "packed_gemv_group.hip": [],
     "packed_gemv_rows.hip": [],
     "token_linear.hip": [],

@@ -315,6 +315,46 @@ __device__ __forceinline__ void write_pair_tables(uint32_t *lds, const float (&l
   }
 }
 
+// The weight half of the block alone (W_ONLY above), for pair tables, without a lane exchange: lane l of
+// wavefront w writes 16-byte chunk l % 8 of rows 8 (w + WAVES i) + l / 8 and loads the two centroids of each
+// of its rows itself, with the kernel's first requests (request_w_rows); an entry is then one conversion.
+template <int BITS, int WAVES> struct WRows {
+  static constexpr int kLevels = 1 << BITS;
+  static constexpr int kRows = kLevels * kLevels < 256 ? kLevels * kLevels : 256;
+  static constexpr int kGroups = kRows / 8;
+  static constexpr int kIters = (kGroups + WAVES - 1) / WAVES;  // at most 8 (four wavefronts, 256 rows)
+};
+
+template <int BITS, int WAVES>
+__device__ __forceinline__ void request_w_rows(float (&lo)[8], float (&hi)[8],
+                                               const float *__restrict__ w_cents) {
+  typedef WRows<BITS, WAVES> W;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < W::kIters; ++i) {
+    const int e = (8 * (wave + WAVES * i) + (lane >> 3)) & (W::kRows - 1);  // (a wavefront past the last group reads a row it does not write)
+    lo[i] = w_cents[e & (W::kLevels - 1)];
+    hi[i] = w_cents[(e >> BITS) & (W::kLevels - 1)];
+  }
+}
+
+template <int BITS, int WAVES>
+__device__ __forceinline__ void write_w_rows(uint32_t *lds, const float (&lo)[8], const float (&hi)[8]) {
+  typedef WRows<BITS, WAVES> W;
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < W::kIters; ++i) {
+    const int grp8 = wave + WAVES * i;
+    if (grp8 >= W::kGroups) break;  // the same for the whole wavefront
+    const f32x2_t pair = {lo[i], hi[i]};
+    const uint32_t d = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
+    *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned char *>(lds) + (8 * grp8 + (lane >> 3)) * 256 + (lane & 7) * 16) =
+        make_uint4(d, d, d, d);
+  }
+}
+
 template <int BITS>
 __device__ __forceinline__ void load_w(const uint8_t *p, uint32_t (&w)[BITS]) {
   if constexpr (BITS == 4) {

@@ -93,8 +93,24 @@ static_assert(kEpiLdsBytes <= kTableBytes, "the epilogue reuses the table block"
 //               ending up with one 32-row slice of the tile, which it scales and stores.  FM = 4.
 // NBUF = K-steps of packed operands held in registers (NBUF-1 of them in flight from memory).
 template <int AM, int BITS, int FM, int FN, int KSPLIT = 1, int NBUF = (FM * FN >= 12 ? 2 : 3)>
-__global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, const float *act_cents, const uint8_t *a_codes,
+                                                          const uint8_t *w_packed, const uint16_t *map_table, int K32, int M32,
+                                                          int N32, int levels_splits, GemmArgs rest) {
   static_assert(KSPLIT == 1 || (KSPLIT == 4 && FM == 4), "K split: four wavefronts, four row slices");
+  // What the first loads need comes as leading scalar arguments: the first fourteen dwords of a kernel's
+  // arguments are handed over in scalar registers when a wavefront starts (the build asks for that with
+  // -mllvm -amdgpu-kernarg-preload-count=16), so centroids and packed operands are requested without
+  // waiting for a load of the argument block; the struct behind them is read for the epilogue's operands.
+  GemmArgs g = rest;
+  g.w_cents = w_cents; g.act_cents = act_cents; g.a = a_codes; g.w = w_packed;
+  g.K = K32; g.M = M32; g.N = N32;
+  g.a_levels = levels_splits & 0xffff; g.k_splits = (levels_splits >> 16) & 0xff; g.window_ahead = (levels_splits >> 24) & 1;
+  g.out_map.table = map_table;
+  {  // (tile counts from the sizes: two divisions by constants instead of two more arguments)
+    constexpr int kTM = (KSPLIT == 1 ? 2 : 1) * FM * 32, kTN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
+    g.tiles_m = (M32 + kTM - 1) / kTM;
+    g.tiles_n = (N32 + kTN - 1) / kTN;
+  }
   __shared__ __attribute__((aligned(65536))) uint32_t lds[kTableBytes / 4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -111,8 +127,8 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   // Loads of one wavefront return in order, and the compiler waits for a load where its value is
   // first touched.  So everything the prologue needs from memory is REQUESTED here, branch-free
   // (indices clamped into the tables, nothing loaded on one side of a branch only), in the order
-  // centroids, epilogue factors, packed operands of the first K-steps, and nothing is looked at
-  // before the last of these requests has been issued: the tables are then written while the
+  // centroids, packed operands of the first K-steps, what only the epilogue needs, and nothing is
+  // looked at before the last of these requests has been issued: the tables are then written while the
   // packed data is still in flight.  (Converting a centroid where it was loaded put one memory
   // round trip per table operand in front of the first operand load of every workgroup.)
   constexpr bool kPairTables = BITS <= 4 && AM != A_U8;  // built without a lane exchange (packed_decode.h)
@@ -139,28 +155,6 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
       a_c0 = a_c1 = g.act_cents[min(tid, g.a_levels - 1)];
     }
   }
-  // The window of an output map (an activation function as a table, gemm_epilogue.h) is requested with
-  // the rest and parked in LDS behind the tables (16 KB of dynamic LDS, which mapped launches ask for),
-  // so that the epilogue finds it there instead of starting with a memory round trip of its own.
-  extern __shared__ __attribute__((aligned(16))) unsigned char map_window[];
-  const bool window_ahead = g.window_ahead != 0;  // uniform
-  // (requested without a branch - a launch without a map reads the first bytes of the weights - and held as
-  // native vectors: an array of the struct type would be pinned in scratch memory)
-  lds_u32x4 window_piece0, window_piece1, window_piece2, window_piece3;
-  {
-    constexpr int kChunksPerSign = (2 << kWideLog2) / 16;
-    const unsigned char *window_from = window_ahead ? reinterpret_cast<const unsigned char *>(g.out_map.table + g.out_map.lo)
-                                                    : reinterpret_cast<const unsigned char *>(g.w);
-    auto piece = [&](int v) {
-      const int i = tid + 256 * v, sign = i / kChunksPerSign, j = i % kChunksPerSign;
-      return *reinterpret_cast<const lds_u32x4 *>(window_from + (window_ahead ? (sign << 16) + 16 * j : 0));
-    };
-    window_piece0 = piece(0);
-    window_piece1 = piece(1);
-    window_piece2 = piece(2);
-    window_piece3 = piece(3);
-  }
-
   constexpr int TM = (KSPLIT == 1 ? 2 : 1) * FM * 32, TN = (KSPLIT == 1 ? 2 : 1) * FN * 32;
   // tile order: spread consecutive workgroup ids over the 8 XCDs' private L2s in
   // contiguous chunks, then walk groups of 4 tile-rows column by column
@@ -185,8 +179,6 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   const int64_t m_base = static_cast<int64_t>(pid_m) * TM + wm;
   const int64_t n_base = static_cast<int64_t>(pid_n) * TN + wn;
 
-  EpiRaw<FM> epi_raw;
-  gemm_epilogue_request<FM>(epi_raw, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.w_cents);
 
   constexpr int kAStep = AM == A_NIBBLE ? 32 : AM == A_U8 ? 64 : AM == A_TILED ? 4096 : 128;  // bytes from one K-step of 64 to the next in a lane's activation stream
   constexpr int kAVec = AM == A_NIBBLE ? 1 : AM == A_U8 ? 2 : 4;        // 16-byte loads per lane per K-step
@@ -255,6 +247,30 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
   fetch(std::integral_constant<int, 0>{}, 0);
   if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
 
+  // behind the operands (a wavefront's loads return in order): what only the epilogue needs
+  // The window of an output map (an activation function as a table, gemm_epilogue.h) is requested with
+  // the rest and parked in LDS behind the tables (16 KB of dynamic LDS, which mapped launches ask for),
+  // so that the epilogue finds it there instead of starting with a memory round trip of its own.
+  extern __shared__ __attribute__((aligned(16))) unsigned char map_window[];
+  const bool window_ahead = g.window_ahead != 0;  // uniform
+  // (requested without a branch - a launch without a map reads the first bytes of the weights - and held as
+  // native vectors: an array of the struct type would be pinned in scratch memory)
+  lds_u32x4 window_piece0, window_piece1, window_piece2, window_piece3;
+  {
+    constexpr int kChunksPerSign = (2 << kWideLog2) / 16;
+    const unsigned char *window_from = window_ahead ? reinterpret_cast<const unsigned char *>(g.out_map.table + kWideLoBf16)  // (the launcher parks windows of this base only)
+                                                    : reinterpret_cast<const unsigned char *>(g.w);
+    auto piece = [&](int v) {
+      const int i = tid + 256 * v, sign = i / kChunksPerSign, j = i % kChunksPerSign;
+      return *reinterpret_cast<const lds_u32x4 *>(window_from + (window_ahead ? (sign << 16) + 16 * j : 0));
+    };
+    window_piece0 = piece(0);
+    window_piece1 = piece(1);
+    window_piece2 = piece(2);
+    window_piece3 = piece(3);
+  }
+
+
   __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a value may be scheduled above the requests
   // (first use of the requested values: every request above has been issued)
 #ifdef OQ_GEMM_STAMPS
@@ -270,6 +286,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(GemmArgs g) {
     const uint32_t my_a = pack16(a_ok0 ? a_c0 : 0.0f, a_ok1 ? a_c1 : 0.0f, false);
     write_row_tables(lds, my_w, my_a);
   }
+  // the epilogue's factors: their addresses come from the argument block in memory, which has arrived by now
+  // (requested with the rest, they would hold the table build back until it had)
+  EpiRaw<FM> epi_raw;
+  gemm_epilogue_request<FM>(epi_raw, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, wm, tid, g.M, g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, g.w_cents);
   if (window_ahead) {
     lds_u32x4 *dst = reinterpret_cast<lds_u32x4 *>(map_window) + tid;
     dst[0] = window_piece0;
@@ -563,9 +583,13 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   const unsigned splits = (KSPLIT == 1 && (AM == A_NIBBLE || AM == A_U8) && g.k_splits > 1) ? static_cast<unsigned>(g.k_splits) : 1u;
   if (splits == 1) g.k_splits = 1;
   // a mapped launch parks the map's window in LDS ahead of its main loop (not for partial tiles: they are not mapped)
-  g.window_ahead = (g.out_map.table != nullptr && g.out_map.lo >= 0 && g.out_dtype == OQ_BF16 && splits == 1 &&
+  g.window_ahead = (g.out_map.table != nullptr && g.out_map.lo == kWideLoBf16 && g.out_dtype == OQ_BF16 && splits == 1 &&
                     reserve_dynamic_lds(reinterpret_cast<const void *>(kern), kWideBytes)) ? 1 : 0;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), g.window_ahead ? kWideBytes : 0, stream, g);
+  if (g.M > 0x7fffffffLL || g.N > 0x7fffffffLL || g.K > 0x7fffffffLL || g.a_levels > 0xffff)
+    return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: a dimension beyond 2^31");
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), g.window_ahead ? kWideBytes : 0, stream,
+                     g.w_cents, g.act_cents, g.a, g.w, g.out_map.table, static_cast<int>(g.K), static_cast<int>(g.M),
+                     static_cast<int>(g.N), g.a_levels | (g.k_splits << 16) | (g.window_ahead << 24), g);
   return check_launch("packed_gemm");
 }
 

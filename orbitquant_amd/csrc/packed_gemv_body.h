@@ -177,10 +177,18 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   uint32_t stage_codes[kStageIters];
   const int stage_groups = ASTAGE ? g.M * static_cast<int>(g.K / 8) : 0;
   uint32_t a_stage = 0;
+  // ... and, with them, the centroids this lane's table rows and its decode of the codes need (vector loads,
+  // branch-free: requested here they arrive with the codes, ahead of the stream; fetched where the
+  // tables are built they were a second memory round trip between the first loads and the first decode)
+  constexpr bool kRowsDirect = ASTAGE && BITS <= 4;
+  float w_row_lo[8], w_row_hi[8];
+  float a_tab_early = 0.0f;
   if constexpr (ASTAGE) {
 #pragma unroll
     for (int i = 0; i < kStageIters; ++i)
       stage_codes[i] = reinterpret_cast<const uint32_t *>(g.a)[min(tid + i * 64 * WAVES, stage_groups - 1)];
+    a_tab_early = g.act_cents[min(lane & 15, g.a_levels - 1)];
+    if constexpr (kRowsDirect) request_w_rows<BITS, WAVES>(w_row_lo, w_row_hi, g.w_cents);
     const uint32_t v0 = static_cast<uint32_t>(min(r, g.M - 1)) * static_cast<uint32_t>(g.K) + 32u * grp;
     a_stage = lds_base + 128u + ((v0 >> 6) << 8) + ((v0 & 63u) << 1);
   }
@@ -265,9 +273,14 @@ __device__ __forceinline__ void packed_gemv_body(const GemvArgs &g, uint32_t *ld
   }
 
   // ---- tables (built while the stream is in flight) ---------------------------------------
-  build_row_tables<BITS, WAVES, BYTES, ASTAGE>(lds, g.w_cents, g.act_cents, g.a_levels);
+  if constexpr (kRowsDirect) {
+    __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a value above the requests
+    write_w_rows<BITS, WAVES>(lds, w_row_lo, w_row_hi);
+  } else {
+    build_row_tables<BITS, WAVES, BYTES, ASTAGE>(lds, g.w_cents, g.act_cents, g.a_levels);
+  }
   if constexpr (ASTAGE) {
-    const float a_tab = lane_table<16>(g.act_cents, g.a_levels);
+    const float a_tab = (lane & 15) < g.a_levels ? a_tab_early : 0.0f;  // centroid l % 16 in lane l (codes past the table read zero)
 #pragma unroll
     for (int i = 0; i < kStageIters; ++i) {
       if (i * 64 * WAVES >= stage_groups) break;  // the same for every thread
