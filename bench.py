@@ -287,6 +287,10 @@ class RawLinear:
         fmt = {"u8": ops.OQ_CODES_U8, "nibble": ops.OQ_CODES_NIBBLE}[self.fmt]
         packed, w_bits, w_cents = layer._matmul_weight(m)   # what the layer's forward reads at this token count
         self.keep = (packed, w_cents)
+        # the workspace the call may use (partial tiles of a launch that shares K between workgroups), allocated once
+        self.ws_bytes = int(self.lib.oq_packed_linear_workspace_bytes(m, n, k, int(w_bits), fmt, int(layer.activation_bits)))
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev) if self.ws_bytes else None
+        self.ws_ptr = None if self.ws is None else self.ws.data_ptr()
         levels = layer._activation_codebook_boundaries.numel() + 1
         imap = layer._input_activation_table
         omap = layer._output_activation_table if with_output_map else None
@@ -313,19 +317,20 @@ class RawLinear:
                          ops._dt(bias) if bias is not None else ops.OQ_F32, n, self.codes.data_ptr(), self.norms.data_ptr(),
                          self.out.data_ptr(), dt, ops._ptr(omap)))
 
-    def _call(self, what):
+    def _call(self, what, workspace):
         fn, args = what   # (the stream is looked up per call: under graph capture it is the capturing stream)
-        if fn(*args, torch.cuda.current_stream().cuda_stream) != 0:
+        tail = (self.ws_ptr, self.ws_bytes) if workspace else ()
+        if fn(*args, *tail, torch.cuda.current_stream().cuda_stream) != 0:
             raise RuntimeError(self.lib.oq_last_error().decode())
 
     def quantize(self):
-        self._call(self._quantize)
+        self._call(self._quantize, False)
 
     def gemm(self):
-        self._call(self._gemm)
+        self._call(self._gemm, True)
 
     def linear(self):
-        self._call(self._linear)
+        self._call(self._linear, True)
         return self.out
 
 
@@ -477,6 +482,10 @@ def copy_calibration(device, launches=3, mib=256):
     torch.cuda.synchronize()
 
 
+TRAFFIC_SOURCE = ("recorded, not measured by this run: profiles/traffic.txt holds the bytes per launch that rocprofv3's "
+                  "FETCH_SIZE and WRITE_SIZE counters gave for this kernel and shape")
+
+
 def recorded_traffic(key: str):
     """HBM bytes per launch of the dominant kernel, measured with the profiler's FETCH_SIZE and WRITE_SIZE
     counters and written down in profiles/ (a live run cannot read those counters itself)."""
@@ -525,7 +534,7 @@ def small_m_roofline(device, iters, m=1, copies=16):
     def fn():
         stream = torch.cuda.current_stream().cuda_stream   # (under graph capture: the capturing stream)
         for c in calls:
-            if lib.oq_packed_linear(*c, stream) != 0:
+            if lib.oq_packed_linear(*c, None, 0, stream) != 0:
                 raise RuntimeError(lib.oq_last_error().decode())
     fn()
     torch.cuda.synchronize()
@@ -534,13 +543,16 @@ def small_m_roofline(device, iters, m=1, copies=16):
     nbytes = mats[0].numel() + 2 * n
     achieved = nbytes / per_launch / 1e9
     return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": recorded_traffic("c5_gemv_w4_4096x14336"), "kernel": "packed_gemv_kernel<4> on 4096->14336 W4",
+            "traffic": recorded_traffic("c5_gemv_w4_4096x14336"), "traffic_source": TRAFFIC_SOURCE, "kernel": "packed_gemv_kernel<4> on 4096->14336 W4",
             "M": m, "bytes_per_launch": nbytes, "avg_launch_us": per_launch * 1e6, "distinct_matrices": copies}
 
 
 def c3_gemm_lines(device, iters):
     """The packed GEMMs of the Flux-style block (c3: W3A3, M = 4608), each timed alone: the other half
-    of "DiT-XL / Flux shapes" of the large-M target, reported beside the c2 headline."""
+    of "DiT-XL / Flux shapes" of the large-M target, reported beside the c2 headline.  The figures are
+    for the layer as it is by default - the stored 3-bit index stream, fields straddling bytes; the
+    `four_bit_copy_*` keys are the same launches on the opt-in copy of the indices at four bits each
+    (`OrbitLinear.nibble_copy_for_many_tokens`, N*K/2 more bytes per layer)."""
     spec = workload_spec("c3", 0)
     gen = torch.Generator().manual_seed(3)
     layers = build_layers(spec, device, gen, False)
@@ -548,9 +560,17 @@ def c3_gemm_lines(device, iters):
     for i, (layer, _act) in enumerate(layers):
         k, n = layer.in_features, layer.out_features
         x = make_input(spec, k, gen).to(device)
+        layer.nibble_copy_for_many_tokens = False
         t = time_kernel(gemm_only_closure(layer, x), max(5, iters // 2))
         tflops = 2.0 * spec["M"] * n * k / t / 1e12
-        out[f"{k}->{n}"] = {"gemm_us": t * 1e6, "gemm_tflops": tflops, "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
+        line = {"gemm_us": t * 1e6, "gemm_tflops": tflops, "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "weights": "stored 3-bit stream"}
+        layer.nibble_copy_for_many_tokens = True
+        t4 = time_kernel(gemm_only_closure(layer, x), max(5, iters // 2))
+        line["four_bit_copy_gemm_us"] = t4 * 1e6
+        line["four_bit_copy_frac"] = 2.0 * spec["M"] * n * k / t4 / 1e12 / MFMA_BF16_PEAK_TFLOPS
+        layer.nibble_copy_for_many_tokens = False
+        layer._nibble_weight_copy = None
+        out[f"{k}->{n}"] = line
     return out
 
 
@@ -695,7 +715,7 @@ def measure_c5(args, device, brief=False):
                       l._activation_codebook_centroids.data_ptr(), 4, l.rotation.block_size, l.activation_eps,
                       l.rotation.normalization, l._rotation_plan.data_ptr(), l.packed_weight_indices.data_ptr(), l.weight_bits,
                       l.row_norms.data_ptr(), l._weight_codebook_centroids.data_ptr(), None, 0, l.out_features,
-                      bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, None, stream))
+                      bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), 2, None, None, 0, stream))
 
     def abi_step():
         fn = lib.oq_quantized_linear
@@ -826,7 +846,7 @@ def main() -> int:
                                   "layer's quantize kernel" if any(l._input_activation_table is not None for l, _ in layers)
                                   else "torch gelu kernel between the linears")},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded_traffic(f"{args.workload}_gemm"),
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": recorded_traffic(f"{args.workload}_gemm"), "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "packed_gemm_kernel" + (" with the GELU table in its epilogue"
                                                        if "gemm_us_without_activation" in dom else ""),
                      "shape_mnk": dom["shape"], "avg_launch_us": dom["gemm_us"]},

@@ -177,9 +177,15 @@ int oq_debug_override(const char *name, const char *value);
  * workgroup), larger M the MFMA tile kernel.  A token row's result does not depend on the
  * rows computed with it as long as the call stays within 64 rows.  A problem with few output
  * tiles and many K-steps (some hundred tokens on a short-and-long matrix) is shared between
- * workgroups along K: fp32 partial tiles go through a device buffer the library keeps per
- * (device, stream) and grows on demand - the one allocation this entry point can make; it is
- * skipped while the stream is being captured and inside oq_quantized_linear_static.
+ * workgroups along K when the caller provides a workspace for the fp32 partial tiles:
+ *
+ * workspace    NULL, or a device buffer of at least oq_packed_linear_workspace_bytes(...) bytes, 16-byte
+ *              aligned, that this call may overwrite (calls on one stream are ordered and may share one).
+ *              The library allocates nothing: as in the reference, whose Python wrapper owns every
+ *              allocation (torch-ext/orbitquant_packed_matmul/__init__.py:130-160), kernels borrow all
+ *              pointers.  NULL, or too small: the single launch.  Which kernel runs depends on the
+ *              arguments alone, so a call captured into a graph computes what the eager call does, bit
+ *              for bit.
  *
  * codes        activation codes in code_format (see oq_rotate_quantize)
  * token_norms  fp32 [M]
@@ -197,7 +203,14 @@ int oq_packed_linear(const void *codes, int code_format, const float *token_norm
                      const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                      const float *w_centroids, const void *bias, int bias_dtype,
                      int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
-                     void *stream);
+                     void *workspace, uint64_t workspace_bytes, void *stream);
+
+/*
+ * Bytes of workspace oq_packed_linear (and _mapped, oq_quantized_linear, and each member of a group)
+ * can make use of for this shape; 0 when it takes a single launch anyway.  No counterpart in the
+ * reference (its wrapper sizes its own temporaries).
+ */
+uint64_t oq_packed_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int w_bits, int code_format, int a_bits);
 
 /*
  * `count` packed linears on the SAME activation codes (the q, k and v projections of an attention
@@ -216,7 +229,8 @@ int oq_packed_linear_group(const void *codes, int code_format, const float *toke
                            const uint8_t *const *packed_w, const int *w_bits,
                            const uint16_t *const *row_norms, const float *const *w_centroids,
                            const void *const *bias, int bias_dtype, int64_t M, const int64_t *N,
-                           int64_t K, void *const *out, int out_dtype, void *stream);
+                           int64_t K, void *const *out, int out_dtype,
+                           void *workspace, uint64_t workspace_bytes, void *stream);
 
 /*
  * oq_packed_linear followed by an elementwise function of the 16-bit outputs given as a
@@ -231,7 +245,7 @@ int oq_packed_linear_mapped(const void *codes, int code_format, const float *tok
                             const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                             const float *w_centroids, const void *bias, int bias_dtype,
                             int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
-                            const uint16_t *output_map, void *stream);
+                            const uint16_t *output_map, void *workspace, uint64_t workspace_bytes, void *stream);
 
 /*
  * The whole quantized-linear forward in one call: oq_rotate_quantize (through
@@ -267,7 +281,8 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map,
                         const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                         const float *w_centroids, const void *bias, int bias_dtype, int64_t N,
                         void *codes_scratch, float *norms_scratch,
-                        void *out, int out_dtype, const uint16_t *output_map, void *stream);
+                        void *out, int out_dtype, const uint16_t *output_map,
+                        void *workspace, uint64_t workspace_bytes, void *stream);
 
 /*
  * oq_quantized_linear for `count` linears that read the same input (q, k and v of an attention
@@ -285,7 +300,8 @@ int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_
                               const uint16_t *const *row_norms, const float *const *w_centroids,
                               const void *const *bias, int bias_dtype, const int64_t *N,
                               void *codes_scratch, float *norms_scratch,
-                              void *const *out, int out_dtype, void *stream);
+                              void *const *out, int out_dtype,
+                              void *workspace, uint64_t workspace_bytes, void *stream);
 
 /*
  * oq_quantized_linear for callers that cannot allocate device memory or bring a workspace:
@@ -322,17 +338,20 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
  * Replaces matmul_packed_weight (torch_binding.cpp:7-12,32-38; packed_matmul.cu:1335-1713).
  * bits in [1, 8].  token_scale: NULL, or fp32 [M] multiplied into row m (lets the
  * caller pass unit-norm bf16 centroids plus token norms).
- * Keeps device memory of its own: bf16 activations (from two tokens on; one token on large matrices) are first
- * rewritten into the matrix core's operand order, into a buffer of 2 * M * K bytes (rows padded to 32)
- * that the library keeps per (device, stream), grows when a larger call comes and releases when the
- * process ends.  Calls on one stream are ordered and share it; while the stream is being captured
- * into a graph the call takes a kernel that needs no buffer.
+ * workspace: NULL, or oq_matmul_packed_weight_workspace_bytes(...) bytes of device memory, 16-byte aligned,
+ * that the call may overwrite.  With it, bf16 activations (from two tokens on; one token on large matrices)
+ * are first rewritten into the matrix core's operand order (2 * M * K bytes, rows padded to 32) and the
+ * tile kernel reads that copy; without it every wavefront stages its own rows through LDS (no buffer, the
+ * same sums, 10-15 % slower on large problems).  The library allocates nothing.
  */
 int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale,
                             const uint8_t *packed_w, int bits, const uint16_t *row_norms,
                             const float *w_centroids, const void *bias, int bias_dtype,
                             int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
-                            void *stream);
+                            void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* Bytes of workspace oq_matmul_packed_weight can make use of for this shape (0: none). */
+uint64_t oq_matmul_packed_weight_workspace_bytes(int64_t M, int64_t N, int64_t K, int w_bits, int x_dtype);
 
 /*
  * Packed INT4 group-scaled linear on bf16 activations (the AdaLN modulation linears):

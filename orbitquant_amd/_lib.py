@@ -21,7 +21,7 @@ _STATUS = {1: "invalid argument", 2: "unsupported", 3: "launch failure"}
 EXPORTS = (
     "oq_device_ok", "oq_last_error", "oq_version", "oq_debug_override", "oq_rotate_quantize", "oq_rotate_plan_bytes", "oq_rotate_plan_build", "oq_quantize_weight", "oq_rotate_quantize_mapped",
     "oq_packed_linear", "oq_packed_linear_group", "oq_packed_linear_mapped", "oq_quantized_linear", "oq_quantized_linear_group", "oq_quantized_linear_static", "oq_matmul_packed_weight", "oq_matmul_packed_adaln_int4", "oq_quantize_adaln_weight", "oq_unpack_lowbit", "oq_pack_lowbit",
-    "oq_dequantize_packed_weight",
+    "oq_dequantize_packed_weight", "oq_packed_linear_workspace_bytes", "oq_matmul_packed_weight_workspace_bytes",
 )
 
 _lib = None
@@ -60,26 +60,31 @@ def load() -> ctypes.CDLL:
     lib.oq_debug_override.restype = c_int
     lib.oq_debug_override.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
     lib.oq_packed_linear.restype = c_int
+    c_u64 = ctypes.c_uint64
     lib.oq_packed_linear.argtypes = [vp, c_int, vp, vp, c_int, vp, c_int, vp, vp, vp, c_int,
-                                     c_i64, c_i64, c_i64, vp, c_int, vp]
+                                     c_i64, c_i64, c_i64, vp, c_int, vp, c_u64, vp]
+    lib.oq_packed_linear_workspace_bytes.restype = c_u64
+    lib.oq_packed_linear_workspace_bytes.argtypes = [c_i64, c_i64, c_i64, c_int, c_int, c_int]
+    lib.oq_matmul_packed_weight_workspace_bytes.restype = c_u64
+    lib.oq_matmul_packed_weight_workspace_bytes.argtypes = [c_i64, c_i64, c_i64, c_int, c_int]
     lib.oq_packed_linear_group.restype = c_int
     lib.oq_packed_linear_group.argtypes = [vp, c_int, vp, vp, c_int, c_int, vp, vp, vp, vp, vp, c_int,
-                                           c_i64, vp, c_i64, vp, c_int, vp]
+                                           c_i64, vp, c_i64, vp, c_int, vp, c_u64, vp]
     lib.oq_packed_linear_mapped.restype = c_int
     lib.oq_packed_linear_mapped.argtypes = [vp, c_int, vp, vp, c_int, vp, c_int, vp, vp, vp, c_int,
-                                            c_i64, c_i64, c_i64, vp, c_int, vp, vp]
+                                            c_i64, c_i64, c_i64, vp, c_int, vp, vp, c_u64, vp]
     lib.oq_quantized_linear.restype = c_int
     lib.oq_quantized_linear.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f, vp,
-                                        vp, c_int, vp, vp, vp, c_int, c_i64, vp, vp, vp, c_int, vp, vp]
+                                        vp, c_int, vp, vp, vp, c_int, c_i64, vp, vp, vp, c_int, vp, vp, c_u64, vp]
     lib.oq_quantized_linear_group.restype = c_int
     lib.oq_quantized_linear_group.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f, vp,
-                                              c_int, vp, vp, vp, vp, vp, c_int, vp, vp, vp, vp, c_int, vp]
+                                              c_int, vp, vp, vp, vp, vp, c_int, vp, vp, vp, vp, c_int, vp, c_u64, vp]
     lib.oq_quantized_linear_static.restype = c_int
     lib.oq_quantized_linear_static.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f, vp,
                                                vp, c_int, vp, vp, vp, c_int, c_i64, vp, c_int, vp, vp]
     lib.oq_matmul_packed_weight.restype = c_int
     lib.oq_matmul_packed_weight.argtypes = [vp, c_int, vp, vp, c_int, vp, vp, vp, c_int,
-                                            c_i64, c_i64, c_i64, vp, c_int, vp]
+                                            c_i64, c_i64, c_i64, vp, c_int, vp, c_u64, vp]
     lib.oq_matmul_packed_adaln_int4.restype = c_int
     lib.oq_matmul_packed_adaln_int4.argtypes = [vp, vp, vp, vp, c_i64, c_i64, c_i64, c_i64, vp, vp]
     lib.oq_quantize_adaln_weight.restype = c_int

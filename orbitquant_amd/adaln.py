@@ -115,9 +115,13 @@ class RTNInt4Linear(nn.Module):
                    scales=torch.zeros(n, groups, dtype=torch.bfloat16, device=device), bias=bias, module_name=module_name)
 
     def _apply(self, fn, recurse: bool = True):
+        # A dtype cast of the model (`.half()`, `.float()`, `pipe.to(torch.float16)`) must not change the stored
+        # format, and must not fail half-way either: the scales are put aside, moved with the rest, and come
+        # back as the bfloat16 values they were (a cast to another dtype and back would round them).
+        kept = self.scales.data
         result = super()._apply(fn, recurse=recurse)
-        if self.scales.dtype != torch.bfloat16:   # a .to(dtype=...) cast must not change the stored format
-            raise RuntimeError("RTNInt4Linear stores its scales as bfloat16; cast activations, not the module")
+        if self.scales.dtype != torch.bfloat16:
+            self.scales.data = kept.to(device=self.scales.device)
         return result
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -62,16 +62,6 @@ void env_load() {
 }
 }  // namespace
 
-namespace {
-thread_local int no_allocation_depth = 0;
-struct NoAllocation {
-  NoAllocation() { ++no_allocation_depth; }
-  ~NoAllocation() { --no_allocation_depth; }
-};
-}  // namespace
-
-bool allocation_forbidden() { return no_allocation_depth > 0; }
-
 // The experiment switches: read from the environment once per process, then only changed through
 // oq_debug_override.
 const char *debug_env(int which) {
@@ -103,7 +93,9 @@ int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const
                          uint16_t *row_norms_out, hipStream_t stream);
 int gemm_tiled_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
                         const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                        int out_dtype, hipStream_t stream);
+                        int out_dtype, void *workspace, uint64_t workspace_bytes, hipStream_t stream);
+uint64_t gemm_tiled_workspace_bytes(int64_t M, int64_t K);
+uint64_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits);
 int gemm_staged_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
                          const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
                          int out_dtype, hipStream_t stream);
@@ -135,7 +127,7 @@ bool gemm_supported(int64_t K, int bits);
 int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                  int out_dtype, const uint16_t *out_map, hipStream_t stream);
+                  int out_dtype, const uint16_t *out_map, void *workspace, uint64_t workspace_bytes, hipStream_t stream);
 int apply_value_map(void *out, int64_t count, const uint16_t *table, hipStream_t stream);
 int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits);
 bool gemm_av_supported(int64_t K, int bits);
@@ -253,7 +245,7 @@ static int packed_linear_impl(const void *codes, int code_format, const float *t
                               const float *act_centroids, int a_bits, const uint8_t *packed_w, int w_bits,
                               const uint16_t *row_norms, const float *w_centroids, const void *bias, int bias_dtype,
                               int64_t M, int64_t N, int64_t K, void *out, int out_dtype, const uint16_t *out_map,
-                              void *stream) {
+                              void *workspace, uint64_t workspace_bytes, void *stream) {
   if (int rc = check_matmul_common("packed_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
   if (M == 0) return OQ_OK;
   if (codes == nullptr || act_centroids == nullptr) return fail(OQ_ERR_INVALID, "packed_linear: null codes/centroids");
@@ -274,7 +266,7 @@ static int packed_linear_impl(const void *codes, int code_format, const float *t
                        bias, bias_dtype, M, N, K, out, out_dtype, s);
   } else if (fast_ptrs && tiled_out && gemm_supported(K, w_bits) && (code_format == OQ_CODES_NIBBLE || M > 16)) {
     return gemm_dispatch(code_format == OQ_CODES_NIBBLE ? 0 : 1, codes, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms, w_centroids,
-                         bias, bias_dtype, M, N, K, out, out_dtype, out_map, s);
+                         bias, bias_dtype, M, N, K, out, out_dtype, out_map, workspace, workspace_bytes, s);
   } else {
     rc = generic_linear_codes(codes, code_format, token_norms, act_centroids, a_levels, packed_w, w_bits, row_norms,
                               w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
@@ -288,19 +280,31 @@ int oq_debug_override(const char *name, const char *value) {
   return debug_env_set(name, value);
 }
 
+uint64_t oq_packed_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int w_bits, int code_format, int a_bits) {
+  if (M <= 0 || N <= 0 || K <= 0 || a_bits < 1 || a_bits > 8) return 0;
+  if (gemv_supported(M, K, w_bits, code_format, 1 << a_bits)) return 0;  // the streaming kernel
+  if (N % 8 != 0 || !gemm_supported(K, w_bits) || !(code_format == OQ_CODES_NIBBLE || M > 16)) return 0;
+  return gemm_workspace_bytes(M, N, K, w_bits);
+}
+
+uint64_t oq_matmul_packed_weight_workspace_bytes(int64_t M, int64_t N, int64_t K, int w_bits, int x_dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || x_dtype != OQ_BF16 || K % 64 != 0 || N % 8 != 0 || !gemm_supported(K, w_bits)) return 0;
+  return gemm_tiled_workspace_bytes(M, K);
+}
+
 int oq_packed_linear(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
                      int a_bits, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms,
                      const float *w_centroids, const void *bias, int bias_dtype, int64_t M, int64_t N,
-                     int64_t K, void *out, int out_dtype, void *stream) {
+                     int64_t K, void *out, int out_dtype, void *workspace, uint64_t workspace_bytes, void *stream) {
   return packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w, w_bits, row_norms,
-                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, nullptr, stream);
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, nullptr, workspace, workspace_bytes, stream);
 }
 
 int oq_packed_linear_group(const void *codes, int code_format, const float *token_norms, const float *act_centroids,
                            int a_bits, int count, const uint8_t *const *packed_w, const int *w_bits,
                            const uint16_t *const *row_norms, const float *const *w_centroids, const void *const *bias,
                            int bias_dtype, int64_t M, const int64_t *N, int64_t K, void *const *out, int out_dtype,
-                           void *stream) {
+                           void *workspace, uint64_t workspace_bytes, void *stream) {
   if (count < 1 || count > 64) return fail(OQ_ERR_INVALID, "packed_linear_group: count=%d (1..64)", count);
   if (packed_w == nullptr || w_bits == nullptr || row_norms == nullptr || w_centroids == nullptr || N == nullptr || out == nullptr)
     return fail(OQ_ERR_INVALID, "packed_linear_group: null argument array");
@@ -321,7 +325,7 @@ int oq_packed_linear_group(const void *codes, int code_format, const float *toke
   for (int i = 0; i < count; ++i)
     if (int rc = packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w[i], w_bits[i],
                                     row_norms[i], w_centroids[i], bias != nullptr ? bias[i] : nullptr, bias_dtype, M,
-                                    N[i], K, out[i], out_dtype, nullptr, stream))
+                                    N[i], K, out[i], out_dtype, nullptr, workspace, workspace_bytes, stream))
       return rc;
   return OQ_OK;
 }
@@ -330,10 +334,10 @@ int oq_packed_linear_mapped(const void *codes, int code_format, const float *tok
                             const float *act_centroids, int a_bits, const uint8_t *packed_w, int w_bits,
                             const uint16_t *row_norms, const float *w_centroids, const void *bias, int bias_dtype,
                             int64_t M, int64_t N, int64_t K, void *out, int out_dtype, const uint16_t *output_map,
-                            void *stream) {
+                            void *workspace, uint64_t workspace_bytes, void *stream) {
   if (output_map == nullptr) return fail(OQ_ERR_INVALID, "packed_linear_mapped: output_map is null");
   return packed_linear_impl(codes, code_format, token_norms, act_centroids, a_bits, packed_w, w_bits, row_norms,
-                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, workspace, workspace_bytes, stream);
 }
 
 int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
@@ -341,7 +345,8 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
                         const float *act_centroids, int a_bits, int64_t block, float eps, float inv_sqrt_block,
                         const void *rotate_plan, const uint8_t *packed_w, int w_bits, const uint16_t *row_norms, const float *w_centroids,
                         const void *bias, int bias_dtype, int64_t N, void *codes_scratch, float *norms_scratch,
-                        void *out, int out_dtype, const uint16_t *output_map, void *stream) {
+                        void *out, int out_dtype, const uint16_t *output_map, void *workspace, uint64_t workspace_bytes,
+                        void *stream) {
   if (int rc = check_matmul_common("quantized_linear", packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
   if (M == 0) return OQ_OK;
   if (a_bits < 1 || a_bits > 8) return fail(OQ_ERR_INVALID, "quantized_linear: a_bits=%d", a_bits);
@@ -366,7 +371,7 @@ int oq_quantized_linear(const void *x, int x_dtype, const uint16_t *input_map, i
                                         input_map, rotate_plan, s))
     return rc;
   return packed_linear_impl(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, packed_w, w_bits, row_norms,
-                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, stream);
+                            w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, output_map, workspace, workspace_bytes, stream);
 }
 
 int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
@@ -375,7 +380,7 @@ int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_
                               const void *rotate_plan, int count, const uint8_t *const *packed_w, const int *w_bits,
                               const uint16_t *const *row_norms, const float *const *w_centroids, const void *const *bias,
                               int bias_dtype, const int64_t *N, void *codes_scratch, float *norms_scratch,
-                              void *const *out, int out_dtype, void *stream) {
+                              void *const *out, int out_dtype, void *workspace, uint64_t workspace_bytes, void *stream) {
   if (count < 1 || count > 64) return fail(OQ_ERR_INVALID, "quantized_linear_group: count=%d (1..64)", count);
   if (packed_w == nullptr || w_bits == nullptr || row_norms == nullptr || w_centroids == nullptr || N == nullptr || out == nullptr)
     return fail(OQ_ERR_INVALID, "quantized_linear_group: null argument array");
@@ -396,7 +401,8 @@ int oq_quantized_linear_group(const void *x, int x_dtype, const uint16_t *input_
                                         input_map, rotate_plan, s))
     return rc;
   return oq_packed_linear_group(codes_scratch, fmt, norms_scratch, act_centroids, a_bits, count, packed_w, w_bits,
-                                row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, stream);
+                                row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, workspace, workspace_bytes,
+                                stream);
 }
 
 int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
@@ -417,16 +423,16 @@ int oq_quantized_linear_static(const void *x, int x_dtype, const uint16_t *input
                 (long long)M, (long long)K, (unsigned long long)(norms_at + 4u * static_cast<uint64_t>(M)), kStaticScratchBytes);
   unsigned char *base = nullptr;
   if (int rc = static_scratch_address(&base)) return rc;
-  NoAllocation guard;  // no launch shape that wants a buffer of the library's own
+  // (no workspace: the launch shapes that need no buffer beyond the scratch)
   return oq_quantized_linear(x, x_dtype, input_map, M, K, perm, signs, boundaries, act_centroids, a_bits, block, eps,
                              inv_sqrt_block, rotate_plan, packed_w, w_bits, row_norms, w_centroids, bias, bias_dtype, N, base,
-                             reinterpret_cast<float *>(base + norms_at), out, out_dtype, output_map, stream);
+                             reinterpret_cast<float *>(base + norms_at), out, out_dtype, output_map, nullptr, 0, stream);
 }
 
 int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale, const uint8_t *packed_w,
                             int bits, const uint16_t *row_norms, const float *w_centroids, const void *bias,
                             int bias_dtype, int64_t M, int64_t N, int64_t K, void *out, int out_dtype,
-                            void *stream) {
+                            void *workspace, uint64_t workspace_bytes, void *stream) {
   if (int rc = check_matmul_common("matmul_packed_weight", packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype)) return rc;
   if (M == 0) return OQ_OK;
   if (x == nullptr || !valid_dtype(x_dtype)) return fail(OQ_ERR_INVALID, "matmul_packed_weight: x / x_dtype");
@@ -440,13 +446,13 @@ int oq_matmul_packed_weight(const void *x, int x_dtype, const float *token_scale
   if (x_dtype == OQ_BF16 && M >= tile_kernel_from && K % 64 == 0 && aligned16(x) && aligned16(packed_w) && gemm_output_ok(N, out) &&
       gemm_supported(K, bits)) {
     // Large M: the tile kernel of the code path on activation values.  Either one pass first puts the activations
-    // into the matrix core's operand order (fastest on large problems; needs a buffer, so not while the stream is
-    // being captured into a graph), or every wavefront stages its own rows through LDS (no buffer).
+    // into the matrix core's operand order (fastest on large problems; needs the caller's workspace), or every
+    // wavefront stages its own rows through LDS (no buffer).
     const char *force = debug_env(ENV_GEMM_TILE);
     const bool force_staged = force != nullptr && force[0] != '\0' && force[1] == 's';
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (!force_staged && hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
-      const int rc = gemm_tiled_dispatch(x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype, s);
+    if (!force_staged) {
+      const int rc = gemm_tiled_dispatch(x, token_scale, packed_w, bits, row_norms, w_centroids, bias, bias_dtype, M, N, K, out, out_dtype,
+                                         workspace, workspace_bytes, s);
       if (rc >= 0) return rc;
     }
     if (M * K * 2 < (int64_t{1} << 32))

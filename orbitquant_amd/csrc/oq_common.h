@@ -18,10 +18,6 @@ int check_launch(const char *what);
 bool reserve_dynamic_lds(const void *kernel, size_t bytes);
 // Experiment switches (environment variables) are read once per process, at first use.
 const char *debug_env(int which);
-// True while the calling thread is inside an entry point that must not allocate
-// (oq_quantized_linear_static): stream_workspace() then hands out nothing, and the dispatchers take
-// the paths that need no buffer.
-bool allocation_forbidden();
 enum DebugEnv { ENV_GEMM_TILE = 0, ENV_NO_TOKEN_LINEAR, ENV_RQ_ONE_GROUP, ENV_GEMV_CFG, ENV_RQ_WAVES, ENV_RQ_FAST_MIN_M, ENV_NO_GEMV_GROUP, ENV_GEMV_GROUP_R, ENV_GEMV_NO_ASTAGE, ENV_GEMV_MAX_M, ENV_GEMM_WG_SPLIT, ENV_FLOAT_GEMM_MIN_M, ENV_GEMM_STAMPS, ENV_COUNT };
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }

@@ -106,10 +106,18 @@ bool gemm_supported(int64_t K, int bits) {
 }
 
 // a_mode: 0 nibble codes, 1 bf16 values, 2 fp16 values
+// Bytes of partial tiles a launch of this shape would like to have (0: it is a single launch anyway).
+uint64_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
+  const int splits = gemm_choose_splits(M, N, K, bits);
+  return splits > 1 ? static_cast<uint64_t>(M) * static_cast<uint64_t>(N) * 4u * static_cast<uint64_t>(splits) : 0u;
+}
+
+// `workspace` (the caller's; NULL or too small: the single launch, whatever the stream is doing) holds the
+// partial tiles of a launch that shares K between workgroups.
 int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float *act_cents, int a_levels,
                   const uint8_t *w, int bits, const uint16_t *row_norms, const float *w_cents,
                   const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                  int out_dtype, const uint16_t *out_map, hipStream_t stream) {
+                  int out_dtype, const uint16_t *out_map, void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
   GemmArgs g{};
   g.a = static_cast<const uint8_t *>(a); g.row_scale = row_scale; g.act_cents = act_cents; g.a_levels = a_levels;
   g.w = w; g.row_norms = row_norms; g.w_cents = w_cents; g.bias = bias; g.bias_dtype = bias_dtype;
@@ -120,15 +128,11 @@ int gemm_dispatch(int a_mode, const void *a, const float *row_scale, const float
   g.k_splits = 1;
   if (const char *where = debug_env(ENV_GEMM_STAMPS)) g.stamps = reinterpret_cast<uint64_t *>(strtoull(where, nullptr, 0));  // builds with -DOQ_GEMM_STAMPS: a device buffer for the kernel's phase stamps
   const int splits = gemm_choose_splits(M, N, K, bits);
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (splits > 1 && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) {
-    // (not while the stream is being captured: the buffer may have to grow)
-    float *partials = static_cast<float *>(stream_workspace(static_cast<size_t>(M) * N * 4 * splits, stream));
-    if (partials != nullptr) {
-      g.k_splits = splits;
-      g.partials = partials;
-      tile = 0;  // 128x128 tiles, two workgroups per CU
-    }
+  if (splits > 1 && workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 &&
+      workspace_bytes >= static_cast<uint64_t>(M) * static_cast<uint64_t>(N) * 4u * static_cast<uint64_t>(splits)) {
+    g.k_splits = splits;
+    g.partials = static_cast<float *>(workspace);
+    tile = 0;  // 128x128 tiles, two workgroups per CU
   }
   const int rc = a_mode == A_NIBBLE ? launch_mode<A_NIBBLE>(g, bits, tile, stream) : gemm_launch_bytes(g, bits, tile, stream);
   if (rc != OQ_OK || g.k_splits == 1) return rc;

@@ -78,7 +78,6 @@ struct GemmArgs {
   uint64_t *stamps;
 };
 
-void *stream_workspace(size_t bytes, hipStream_t stream);  // packed_gemm_tiled.hip
 
 namespace {
 

@@ -4,8 +4,6 @@
 // straight into registers, 1 KB of consecutive bytes per wavefront load, and only the weights go
 // through the lookup tables: 4 FN lookups per FM*FN MFMAs instead of 4 (FM + FN), and no
 // workgroup-wide staging of an activation slab between barriers.
-#include <map>
-#include <mutex>
 #include <utility>
 
 #include "packed_gemm_kernel.h"
@@ -45,49 +43,24 @@ int launch_tiled(const GemmArgs &g, int tile, hipStream_t stream) {
 
 }  // namespace
 
-// A device buffer per (device, stream), grown on demand and kept: work on one stream is ordered, so
-// a later call may reuse what an earlier one has finished with.  NULL when it cannot be had.
-namespace {
-struct Workspace {
-  void *ptr = nullptr;
-  size_t bytes = 0;
-};
-
-}  // namespace
-
-void *stream_workspace(size_t bytes, hipStream_t stream) {
-  static std::mutex lock;
-  static std::map<std::pair<int, hipStream_t>, Workspace> spaces;
-  if (allocation_forbidden()) return nullptr;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> guard(lock);
-  Workspace &w = spaces[std::make_pair(dev, stream)];
-  if (w.bytes >= bytes) return w.ptr;
-  if (w.ptr != nullptr) (void)hipFree(w.ptr);  // waits for the work that still reads it
-  w.ptr = nullptr;
-  w.bytes = 0;
-  const size_t want = bytes + bytes / 4;
-  if (hipMalloc(&w.ptr, want) != hipSuccess) {
-    (void)hipGetLastError();
-    w.ptr = nullptr;
-    return nullptr;
-  }
-  w.bytes = want;
-  return w.ptr;
-}
-
 int gemm_choose_tile(int64_t M, int64_t N, int64_t K, int bits);  // packed_gemm.hip
 
-// x: bf16 [M, K], 16-byte aligned rows (K % 64 == 0).  Under stream capture the caller takes another kernel
-// (the buffer may have to grow, and an allocation is not something to record into a graph).
+// Bytes of the operand-order copy of [M, K] bf16 activations (whole row tiles of 32).
+uint64_t gemm_tiled_workspace_bytes(int64_t M, int64_t K) {
+  const int64_t row_tiles = (M + 31) / 32, pieces = row_tiles * (K / 64) * 256;
+  return row_tiles > 65535 ? 0u : static_cast<uint64_t>(pieces) * 16u;
+}
+
+// x: bf16 [M, K], 16-byte aligned rows (K % 64 == 0).  `workspace`: the caller's buffer for the operand-order
+// copy, gemm_tiled_workspace_bytes(M, K) bytes, 16-byte aligned; -1 (the caller takes the kernel that needs no
+// buffer) when it is absent or too small.
 int gemm_tiled_dispatch(const void *x, const float *token_scale, const uint8_t *w, int bits, const uint16_t *row_norms,
                         const float *w_cents, const void *bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void *out,
-                        int out_dtype, hipStream_t stream) {
-  const int64_t row_tiles = (M + 31) / 32, pieces = row_tiles * (K / 64) * 256;
-  void *tiled = stream_workspace(static_cast<size_t>(pieces) * 16, stream);
-  if (tiled == nullptr) return -1;  // the caller falls back
-  if (row_tiles > 65535) return -1;
+                        int out_dtype, void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
+  const int64_t row_tiles = (M + 31) / 32;
+  const uint64_t need = gemm_tiled_workspace_bytes(M, K);
+  void *tiled = workspace;
+  if (tiled == nullptr || need == 0 || workspace_bytes < need || (reinterpret_cast<uintptr_t>(tiled) & 15u) != 0) return -1;
   hipLaunchKernelGGL(tile_activations_kernel, dim3(static_cast<unsigned>((K / 64 + 3) / 4), static_cast<unsigned>(row_tiles)), dim3(256), 0, stream,
                      static_cast<const uint16_t *>(x), M, K, static_cast<uint4 *>(tiled));
   int rc = check_launch("tile_activations");

@@ -197,11 +197,17 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
   unsigned char *stage = smem + kStageAt;
   const uint32_t *gather = reinterpret_cast<const uint32_t *>(a.plan + plan::kGatherOffset) + (DT == OQ_F32 ? K : 0);
 
-  // A plan built for another shape must not be walked: nothing is written then.  (The gather
-  // entries are absolute LDS addresses, valid because this kernel's LDS block starts at 0.)
+  // A plan built for another shape must not be walked.  No codes are written then, and the row's norm
+  // is stored as NaN, so that the mismatch cannot pass for a result: every output computed from it is NaN.
+  // (The gather entries are absolute LDS addresses, valid because this kernel's LDS block starts at 0.)
   if (hdr->magic != plan::kMagic || hdr->K != static_cast<uint32_t>(K) || hdr->block != static_cast<uint32_t>(H) ||
-      hdr->levels != static_cast<uint32_t>(a.levels) || lds_byte_address(smem) != 0u)
+      hdr->levels != static_cast<uint32_t>(a.levels) || lds_byte_address(smem) != 0u) {
+    if (tid == 0) {
+      if (a.norms != nullptr) a.norms[row] = __builtin_nanf("");
+      if constexpr (EMIT == EMIT_WEIGHT) a.norms_bf16[row] = 0x7fc0;
+    }
     return;
+  }
   const float cell_scale = hdr->cell_scale, cell_offset = hdr->cell_offset;
 
   // tables: entry tid is requested now and stored to LDS after the row has been requested (loads

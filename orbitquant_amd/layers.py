@@ -139,11 +139,14 @@ class OrbitLinear(nn.Module):
         # share its quantization: set this on each of them and the codes the first one computes serve the
         # others (see _shared_codes).  Off by default: the reference quantizes per layer.
         self.share_input_quantization = False
-        # 2- and 3-bit weights, many tokens: the tile kernel reads a copy of the indices repacked at four
-        # bits each (see _matmul_weight).  The copy is made on first need and costs out*in/2 bytes.
-        self.nibble_copy_for_many_tokens = True
+        # 2- and 3-bit weights, many tokens: the tile kernel can read a copy of the indices repacked at four
+        # bits each (see _matmul_weight), 7-17 % faster there.  OFF by default, because the copy costs
+        # out*in/2 bytes on top of the stored stream: a 2-bit layer then holds 0.75 instead of 0.25 byte per
+        # weight (3x), a 3-bit layer 0.875 instead of 0.375 (2.3x) - most of what low-bit weights save.
+        self.nibble_copy_for_many_tokens = False
         self.register_buffer("_nibble_weight_copy", None, persistent=False)
         self.register_buffer("_nibble_weight_centroids", None, persistent=False)
+        self._nibble_copy_of = None   # (address, version) of the packed_weight_indices the copy was made from
 
     MANY_TOKENS = 65   # from here on the matmul is the tile kernel (up to 64 tokens: the streaming kernel)
 
@@ -160,6 +163,13 @@ class OrbitLinear(nn.Module):
             cents = torch.zeros(16, dtype=torch.float32, device=indices.device)
             cents[: 1 << self.weight_bits] = self._weight_codebook_centroids
             self._nibble_weight_centroids = cents
+            self._nibble_copy_of = self._stored_stream_identity()
+
+    def _stored_stream_identity(self):
+        """What tells one state of the stored index stream from another: its address and torch's version
+        counter (None for the counter of an inference tensor, which has none: the address alone then)."""
+        w = self.packed_weight_indices
+        return (w.data_ptr(), None if w.is_inference() else w._version)
 
     def _matmul_weight(self, tokens: int):
         """(packed indices, bits per index, centroids) the matmul of `tokens` rows reads.  The stored
@@ -171,8 +181,10 @@ class OrbitLinear(nn.Module):
         take the streaming kernel, which is bound by decode work per byte, and keep reading the stored stream."""
         if (self.weight_bits in (2, 3) and self.nibble_copy_for_many_tokens and tokens >= self.MANY_TOKENS
                 and self.packed_weight_indices.device.type == "cuda"):
-            if self._nibble_weight_copy is None and not torch.compiler.is_compiling():
-                self.prepare_many_token_weights()
+            if not torch.compiler.is_compiling():   # (a forward being traced neither checks nor builds the copy)
+                stale = self._nibble_weight_copy is not None and self._nibble_copy_of != self._stored_stream_identity()
+                if self._nibble_weight_copy is None or stale:
+                    self.prepare_many_token_weights()   # (also after an in-place update of the stored stream)
             if self._nibble_weight_copy is not None:
                 return self._nibble_weight_copy, 4, self._nibble_weight_centroids
         return self.packed_weight_indices, self.weight_bits, self._weight_codebook_centroids
@@ -312,20 +324,32 @@ class OrbitLinear(nn.Module):
         address, shape, dtype and version counter), quantized by the same rotation and codebook, skips
         its quantizer.  Same kernels as the fused op, so the same output bits.  The entry holds a
         reference to the input, so its address cannot be handed to another tensor meanwhile; writes
-        to the input that bypass torch's version counter are not seen."""
+        to the input that bypass torch's version counter (a raw-pointer kernel refilling a static buffer)
+        are not seen: such callers use `OrbitLinearGroup`, which shares by construction.  Inputs created
+        under `torch.inference_mode()` and calls on a capturing stream are never served from the entry."""
         fmt = "nibble" if self.activation_bits <= 4 else "u8"
-        key = (x.data_ptr(), x._version, tuple(x.shape), x.dtype, x.device, self.in_features, self.rotation.seed,
+        # The entry is reused only when nothing can have changed unseen: an inference tensor has no version
+        # counter (asking for it raises), and a stream under capture replays later on other contents, so
+        # both always quantize; strides and the stream are part of the key (codes made on one stream
+        # are not handed to another without an event).
+        stream = torch.cuda.current_stream(x.device)
+        cacheable = not x.is_inference() and not torch.cuda.is_current_stream_capturing()
+        key = (x.data_ptr(), x._version if cacheable else None, tuple(x.shape), tuple(x.stride()), x.dtype, x.device,
+               stream.cuda_stream, self.in_features, self.rotation.seed,
                self.rotation.block_size, self.activation_bits, self.activation_eps,
                None if table is None else table.data_ptr())
         entry = _last_quantization
-        if entry.get("key") == key:
+        if cacheable and entry.get("key") == key:
             codes, norms = entry["codes"], entry["norms"]
         else:
             codes, _, norms = ops.rotate_quantize(
                 x, self._rotation_permutation, self._rotation_signs, self._activation_codebook_boundaries,
                 block_size=self.rotation.block_size, eps=self.activation_eps, inv_sqrt_block=self.rotation.normalization,
                 code_format=fmt, input_map=table, plan=self._rotation_plan)
-            entry.update(key=key, codes=codes, norms=norms, keep=x)
+            if cacheable:
+                entry.update(key=key, codes=codes, norms=norms, keep=x)
+            else:
+                entry.clear()
         bias = self.bias
         if bias is not None and bias.dtype != x.dtype:
             bias = bias.to(x.dtype)   # as the fused op (and the reference on accelerators) does

@@ -52,6 +52,17 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _workspace(nbytes: int, like: torch.Tensor) -> tuple[int | None, int, torch.Tensor | None]:
+    """(address, size, tensor) of a workspace of `nbytes` for one call, from torch's caching allocator (the
+    library allocates nothing: this wrapper owns allocation, as the reference's does).  The tensor is returned
+    so that the caller keeps it alive until its call has been issued; stream-ordered reuse by the allocator
+    makes it safe to drop then."""
+    if nbytes <= 0:
+        return None, 0, None
+    buf = torch.empty(int(nbytes), dtype=torch.uint8, device=like.device)
+    return buf.data_ptr(), int(nbytes), buf
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -92,6 +103,7 @@ def rotate_plan(permutation: torch.Tensor, signs: torch.Tensor, boundaries: torc
                                       boundaries.numel() + 1, dim, int(block_size), float(inv_sqrt_block),
                                       plan.data_ptr(), _stream(permutation))
     _lib.check(rc, "oq_rotate_plan_build")
+    plan._oq_plan_of = (int(dim), int(block_size), int(boundaries.numel() + 1))
     return plan
 
 
@@ -128,10 +140,21 @@ def quantize_weight(weight: torch.Tensor, permutation: torch.Tensor, signs: torc
     return packed, norms
 
 
-def _plan_operand(plan: torch.Tensor | None, like: torch.Tensor, dim: int) -> torch.Tensor | None:
+def _plan_operand(plan: torch.Tensor | None, like: torch.Tensor, dim: int, block: int | None = None,
+                  levels: int | None = None) -> torch.Tensor | None:
+    """The plan as an operand.  Its byte count depends on the dimension alone, so a plan of another layer
+    with the same dimension would pass that check: `rotate_plan` notes what a plan was built for on the
+    tensor it returns, and a plan carrying such a note is refused here when block or levels differ.  (A
+    plan without the note - a copy, a tensor the caller filled - is checked by the kernel, which stores
+    NaN norms for a plan that does not match its launch.)"""
     if plan is None:
         return None
     expected = int(_lib.load().oq_rotate_plan_bytes(dim))
+    made_for = getattr(plan, "_oq_plan_of", None)
+    if made_for is not None:
+        want = (int(dim), made_for[1] if block is None else int(block), made_for[2] if levels is None else int(levels))
+        if tuple(made_for) != want:
+            raise ValueError(f"this rotate plan was built for (dim, block, levels) = {tuple(made_for)}, the call has {want}")
     return _operand(plan, "plan", like, dtype=torch.uint8, numel=expected)
 
 
@@ -200,7 +223,7 @@ def rotate_quantize(
         if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device:
             raise ValueError("input_map must hold 65536 entries of x's dtype on x's device")
         input_map = input_map.contiguous()
-    plan = _plan_operand(plan, x, dim)
+    plan = _plan_operand(plan, x, dim, block_size, levels)
     lib = _lib.load()
     head = (m, dim, permutation.data_ptr(), signs.data_ptr(), boundaries.data_ptr(), _ptr(centroids), levels,
             int(block_size), float(eps), float(inv_sqrt_block))
@@ -275,11 +298,14 @@ def packed_linear(
             row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
             _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
             out.data_ptr(), _DTYPES[output_dtype])
+    ws_ptr, ws_bytes, ws = _workspace(lib.oq_packed_linear_workspace_bytes(m, int(out_features), int(in_features), int(weight_bits),
+                                                                            fmt, int(activation_bits)), codes)
     with _OnDevice(codes):
         if output_map is None:
-            rc = lib.oq_packed_linear(*args, _stream(codes))
+            rc = lib.oq_packed_linear(*args, ws_ptr, ws_bytes, _stream(codes))
         else:
-            rc = lib.oq_packed_linear_mapped(*args, output_map.data_ptr(), _stream(codes))
+            rc = lib.oq_packed_linear_mapped(*args, output_map.data_ptr(), ws_ptr, ws_bytes, _stream(codes))
+    del ws
     _lib.check(rc, "oq_packed_linear")
     return out.reshape(*lead, out_features)
 
@@ -331,6 +357,9 @@ def packed_linear_group(
     count = len(keep)
     ptrs = ctypes.c_void_p * count
     lib = _lib.load()
+    fmt_code = {"u8": OQ_CODES_U8, "nibble": OQ_CODES_NIBBLE}[code_format]
+    ws_ptr, ws_bytes, ws = _workspace(max(lib.oq_packed_linear_workspace_bytes(m, k[4], int(in_features), k[3], fmt_code, int(activation_bits))
+                                          for k in keep), codes)   # members run one after the other and share it
     with _OnDevice(codes):
         rc = lib.oq_packed_linear_group(
             flat.data_ptr(), fmt, norms.data_ptr(), activation_centroids.data_ptr(), int(activation_bits), count,
@@ -338,7 +367,8 @@ def packed_linear_group(
             ptrs(*[k[1].data_ptr() for k in keep]), ptrs(*[k[2].data_ptr() for k in keep]),
             ptrs(*[_ptr(k[5]) for k in keep]), _DTYPES[bias_dtype] if bias_dtype is not None else OQ_F32, m,
             (ctypes.c_int64 * count)(*[k[4] for k in keep]), int(in_features),
-            ptrs(*[o.data_ptr() for o in outs]), _DTYPES[output_dtype], _stream(codes))
+            ptrs(*[o.data_ptr() for o in outs]), _DTYPES[output_dtype], ws_ptr, ws_bytes, _stream(codes))
+    del ws
     _lib.check(rc, "oq_packed_linear_group")
     return [o.reshape(*lead, o.shape[-1]) for o in outs]
 
@@ -389,19 +419,22 @@ def quantized_linear(
             raise ValueError("output_map must hold 65536 entries of the 16-bit output dtype on x's device")
         output_map = output_map.contiguous()
     bias = _operand(bias, "bias", x, dtype=_FLOATS, numel=out_features)
-    plan = _plan_operand(plan, x, dim)
+    plan = _plan_operand(plan, x, dim, block_size, 1 << activation_bits)
     nibble = activation_bits <= 4 and dim % 2 == 0
     codes = torch.empty((m, dim // 2 if nibble else dim), dtype=torch.uint8, device=x.device)
     norms = torch.empty(m, dtype=torch.float32, device=x.device)
     out = torch.empty((m, out_features), dtype=x.dtype, device=x.device)
     lib = _lib.load()
+    ws_ptr, ws_bytes, ws = _workspace(lib.oq_packed_linear_workspace_bytes(
+        m, int(out_features), dim, int(weight_bits), OQ_CODES_NIBBLE if nibble else OQ_CODES_U8, int(activation_bits)), x)
     with _OnDevice(x):
         rc = lib.oq_quantized_linear(
             rows.data_ptr(), _dt(rows), _ptr(input_map), m, dim, permutation.data_ptr(), signs.data_ptr(),
             boundaries.data_ptr(), act_centroids.data_ptr(), int(activation_bits), int(block_size), float(eps),
             float(inv_sqrt_block), _ptr(plan), packed_weight.data_ptr(), int(weight_bits), row_norms.data_ptr(),
             weight_centroids.data_ptr(), _ptr(bias), _dt(bias) if bias is not None else 0, out_features,
-            codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _ptr(output_map), _stream(x))
+            codes.data_ptr(), norms.data_ptr(), out.data_ptr(), _dt(out), _ptr(output_map), ws_ptr, ws_bytes, _stream(x))
+    del ws
     _lib.check(rc, "oq_quantized_linear")
     return out.reshape(*x.shape[:-1], out_features)
 
@@ -441,7 +474,7 @@ def quantized_linear_group(
         if input_map.dtype != x.dtype or input_map.numel() != 65536 or input_map.device != x.device or x.dtype == torch.float32:
             raise ValueError("input_map must hold 65536 entries of x's 16-bit dtype on x's device")
         input_map = input_map.contiguous()
-    plan = _plan_operand(plan, x, dim)
+    plan = _plan_operand(plan, x, dim, block_size, 1 << activation_bits)
     keep, outs, bias_dtype = [], [], None
     for packed, row_norms, cents, bits, n, bias in weights:
         expected = (n * dim * bits + 7) // 8
@@ -461,6 +494,8 @@ def quantized_linear_group(
     count = len(keep)
     ptrs = ctypes.c_void_p * count
     lib = _lib.load()
+    ws_ptr, ws_bytes, ws = _workspace(max(lib.oq_packed_linear_workspace_bytes(
+        m, k[4], dim, k[3], OQ_CODES_NIBBLE if nibble else OQ_CODES_U8, int(activation_bits)) for k in keep), x)
     with _OnDevice(x):
         rc = lib.oq_quantized_linear_group(
             rows.data_ptr(), _dt(rows), _ptr(input_map), m, dim, permutation.data_ptr(), signs.data_ptr(),
@@ -470,7 +505,8 @@ def quantized_linear_group(
             ptrs(*[k[1].data_ptr() for k in keep]), ptrs(*[k[2].data_ptr() for k in keep]),
             ptrs(*[_ptr(k[5]) for k in keep]), _DTYPES[bias_dtype] if bias_dtype is not None else OQ_F32,
             (ctypes.c_int64 * count)(*[k[4] for k in keep]), codes.data_ptr(), norms.data_ptr(),
-            ptrs(*[o.data_ptr() for o in outs]), _dt(x), _stream(x))
+            ptrs(*[o.data_ptr() for o in outs]), _dt(x), ws_ptr, ws_bytes, _stream(x))
+    del ws
     _lib.check(rc, "oq_quantized_linear_group")
     return [o.reshape(*x.shape[:-1], o.shape[-1]) for o in outs]
 
@@ -501,12 +537,15 @@ def matmul_packed_weight_values(
     token_scale = _operand(token_scale, "token_scale", x, dtype=torch.float32, numel=m)
     out = torch.empty((m, out_features), dtype=out_dtype, device=x.device)
     lib = _lib.load()
+    ws_ptr, ws_bytes, ws = _workspace(lib.oq_matmul_packed_weight_workspace_bytes(m, int(out_features), int(in_features), int(bits),
+                                                                                   _dt(x)), x)
     with _OnDevice(x):
         rc = lib.oq_matmul_packed_weight(
             flat.data_ptr(), _dt(flat), _ptr(token_scale), packed_weight_indices.data_ptr(), int(bits),
             row_norms.data_ptr(), weight_centroids.data_ptr(), _ptr(bias),
             _dt(bias) if bias is not None else OQ_F32, m, int(out_features), int(in_features),
-            out.data_ptr(), _DTYPES[out_dtype], _stream(x))
+            out.data_ptr(), _DTYPES[out_dtype], ws_ptr, ws_bytes, _stream(x))
+    del ws
     _lib.check(rc, "oq_matmul_packed_weight")
     return out.reshape(*lead, out_features)
 

@@ -246,3 +246,22 @@ def test_checksums_are_verified(tmp_path):
         fh.write(b"\0")
     with pytest.raises(RuntimeError, match="checksum mismatch"):
         load_artifact(Tiny(), tmp_path)
+
+
+def test_adaln_module_survives_dtype_casts_of_the_model():
+    """`model.half()` / `.float()` on a model that holds an RTNInt4Linear: no exception, nothing left
+    half-converted; the scales stay the bfloat16 values they were, bias follows the cast like any parameter."""
+    import torch
+    from torch import nn
+
+    from orbitquant_amd import OrbitQuantConfig, RTNInt4Linear
+
+    torch.manual_seed(5)
+    layer = RTNInt4Linear.from_linear(nn.Linear(130, 24), config=OrbitQuantConfig())
+    model = nn.Sequential(nn.LayerNorm(130), layer)
+    scales, packed = layer.scales.detach().clone(), layer.packed_weight.detach().clone()
+    for cast in (model.half, model.float, lambda: model.to(torch.float16), model.bfloat16):
+        cast()
+        assert layer.scales.dtype == torch.bfloat16 and torch.equal(layer.scales, scales)
+        assert layer.packed_weight.dtype == torch.uint8 and torch.equal(layer.packed_weight, packed)
+    assert model[0].weight.dtype == torch.bfloat16 and layer.bias.dtype == torch.bfloat16

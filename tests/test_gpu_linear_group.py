@@ -263,7 +263,7 @@ def test_group_argument_checks(dev):
             c["codes"].data_ptr(), fmt, c["norms"].data_ptr(), c["cents"].data_ptr(), a_bits, count,
             ptrs(*[w[0].data_ptr() for w in c["weights"]]), (ctypes.c_int * 2)(*w_bits),
             ptrs(*[w[1].data_ptr() for w in c["weights"]]), ptrs(*[w[2].data_ptr() for w in c["weights"]]), None, 0, 1,
-            (ctypes.c_int64 * 2)(32, 32), 256, out if out is not None else ptrs(*[o.data_ptr() for o in outs]), 2, None)
+            (ctypes.c_int64 * 2)(32, 32), 256, out if out is not None else ptrs(*[o.data_ptr() for o in outs]), 2, None, 0, None)
 
     assert call() == 0
     assert call(count=0) == 1 and b"count" in lib.oq_last_error()

@@ -53,8 +53,37 @@ def test_copy_gives_the_outputs_of_the_stored_stream(dev, k, n, wbits, abits, m)
         assert (got.float() - want.float()).abs().max().item() <= scale * 2.0 ** -7
 
 
+def test_copy_is_opt_in(dev):
+    """By default a 2- or 3-bit layer keeps its stored stream only: no second copy of the indices."""
+    layer = make_layer(dev, 1024, 512, 3, 4)
+    assert layer.nibble_copy_for_many_tokens is False
+    layer(torch.randn(256, 1024, device=dev, dtype=torch.bfloat16))
+    assert layer._nibble_weight_copy is None and layer._matmul_weight(4096)[1] == 3
+
+
+def test_copy_follows_an_in_place_update(dev):
+    """Indices written in place (same storage, version counter moved): the copy is rebuilt from them."""
+    layer = make_layer(dev, 1024, 512, 3, 4)
+    layer.nibble_copy_for_many_tokens = True
+    other = make_layer(dev, 1024, 512, 3, 4, seed=9)
+    many = torch.randn(256, 1024, device=dev, dtype=torch.bfloat16)
+    first = layer(many)
+    assert layer._nibble_weight_copy is not None
+    with torch.no_grad():
+        layer.packed_weight_indices.copy_(other.packed_weight_indices)
+        layer.row_norms.copy_(other.row_norms)
+        layer.bias.copy_(other.bias)
+    second = layer(many)
+    assert torch.equal(second, other(many)) and not torch.equal(second, first)
+    assert layer._matmul_weight(256)[1] == 4   # and it is a copy of the new indices
+    from orbitquant_amd import ops
+    assert torch.equal(ops.unpack_lowbit(layer._nibble_weight_copy, 4, 512 * 1024),
+                       ops.unpack_lowbit(other.packed_weight_indices, 3, 512 * 1024))
+
+
 def test_copy_follows_the_weights(dev):
     layer = make_layer(dev, 1024, 512, 3, 4)
+    layer.nibble_copy_for_many_tokens = True
     small, many = torch.randn(16, 1024, device=dev, dtype=torch.bfloat16), torch.randn(256, 1024, device=dev, dtype=torch.bfloat16)
     layer(small)
     assert layer._nibble_weight_copy is None                  # decode-sized calls read the stored stream
@@ -74,20 +103,24 @@ def test_copy_follows_the_weights(dev):
     layer.to(dev)
     assert torch.equal(layer(many), second) and layer._nibble_weight_centroids.dtype == torch.float32
     four = make_layer(dev, 1024, 512, 4, 4)
+    four.nibble_copy_for_many_tokens = True
     four(many)
     assert four._nibble_weight_copy is None and four._matmul_weight(4096)[1] == 4
     six = make_layer(dev, 512, 64, 6, 6)
+    six.nibble_copy_for_many_tokens = True
     six(torch.randn(300, 512, device=dev, dtype=torch.bfloat16))
     assert six._nibble_weight_copy is None
 
 
 def test_prepared_copy_under_compile(dev):
     layer = make_layer(dev, 1024, 256, 3, 3)
+    layer.nibble_copy_for_many_tokens = True
     x = torch.randn(384, 1024, device=dev, dtype=torch.bfloat16)
     want = layer(x)                      # builds the copy
     compiled = torch.compile(layer, fullgraph=True)
     assert torch.equal(compiled(x), want)
     fresh = make_layer(dev, 1024, 256, 3, 3)
+    fresh.nibble_copy_for_many_tokens = True
     compiled_fresh = torch.compile(fresh, fullgraph=True)
     out = compiled_fresh(x)              # no copy yet and none can be built while tracing: the stored stream
     assert torch.equal(out, want) or (out.float() - want.float()).abs().max().item() <= want.float().abs().max().item() * 2.0 ** -7

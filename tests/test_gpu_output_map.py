@@ -112,8 +112,8 @@ def test_packed_linear_mapped_entry_point(dev):
     out = torch.empty(200, 256, dtype=torch.float32, device=dev)
     args = (codes.data_ptr(), 1, norms.data_ptr(), c["cents"].data_ptr(), 4, c["packed"].data_ptr(), 4, c["rn"].data_ptr(),
             c["wcents"].data_ptr(), None, 0, 200, 256, 512, out.data_ptr())
-    assert lib.oq_packed_linear_mapped(*args, 0, table.data_ptr(), None) == 1      # fp32 output
-    assert lib.oq_packed_linear_mapped(*args, 2, None, None) == 1                  # null table
+    assert lib.oq_packed_linear_mapped(*args, 0, table.data_ptr(), None, 0, None) == 1      # fp32 output
+    assert lib.oq_packed_linear_mapped(*args, 2, None, None, 0, None) == 1                  # null table
     torch.cuda.synchronize()
 
 

@@ -379,9 +379,10 @@ def test_packed_linear_k_shared_between_workgroups(dev, m, n, k, wbits, abits, s
     check_outputs(fp32, oracle_linear(layer, codes, s, torch.float32), s, layer["r"].float().numpy(), k, "fp32 out")
 
 
-def test_packed_linear_shared_k_is_skipped_under_graph_capture(dev, library_switch):
-    """A captured stream gets the single launch (the buffer of partial tiles may have to grow, which a graph cannot
-    record): the replay returns the bits of the eager single launch."""
+def test_packed_linear_shares_k_under_graph_capture_too(dev, library_switch):
+    """Which kernel a call takes depends on its arguments alone (the partial tiles live in a workspace the
+    caller provides, here the wrapper, from torch's allocator): a captured call shares K like the eager one,
+    and every replay returns the eager call's bits."""
     rng = np.random.default_rng(5)
     m, n, k = 128, 256, 8192
     layer = make_layer(rng, n, k, 4, 4)
@@ -406,11 +407,66 @@ def test_packed_linear_shared_k_is_skipped_under_graph_capture(dev, library_swit
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out = ops.packed_linear(*args, **kw)
-    for _ in range(2):
+    for _ in range(3):
         out.zero_()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(out, single)
+        assert torch.equal(out, split)
+        assert torch.equal(ops.packed_linear(*args, **kw), split)   # eager work between the replays
+
+
+def test_workspace_is_the_callers_and_optional(dev, library_switch):
+    """The C ABI allocates nothing.  Without a workspace (NULL, or one that is too small) oq_packed_linear is the
+    single launch and oq_matmul_packed_weight stages activation rows through LDS; with the bytes the query
+    functions name they share K between workgroups / read an operand-order copy.  Same results as the wrapper's."""
+    from orbitquant_amd import _lib, ops
+
+    lib = _lib.load()
+    rng = np.random.default_rng(6)
+    m, n, k = 128, 256, 8192
+    layer = make_layer(rng, n, k, 4, 4)
+    _, x32 = make_x(rng, m, k, torch.bfloat16)
+    codes, s = oracle_c.rotate_quantize(x32, layer["perm"], layer["signs"], layer["ba"], layer["block"], 1e-10, layer["inv"])
+    library_switch("OQ_GEMM_WG_SPLIT", "1")
+    single = run_packed_linear(dev, layer, codes, s, "nibble")
+    library_switch("OQ_GEMM_WG_SPLIT", "8")
+    split = run_packed_linear(dev, layer, codes, s, "nibble")
+    t = dict(codes=torch.from_numpy(o.pack_nibbles(codes)).to(dev), s=torch.from_numpy(s).to(dev), ca=torch.from_numpy(layer["ca"]).to(dev),
+             packed=torch.from_numpy(layer["packed"]).to(dev), r=layer["r"].to(dev), cw=torch.from_numpy(layer["cw"]).to(dev),
+             bias=torch.from_numpy(layer["bias"]).to(torch.bfloat16).to(dev))
+    need = int(lib.oq_packed_linear_workspace_bytes(m, n, k, 4, 1, 4))
+    assert need == m * n * 4 * 8
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+
+    def call(ws_ptr, ws_bytes):
+        rc = lib.oq_packed_linear(t["codes"].data_ptr(), 1, t["s"].data_ptr(), t["ca"].data_ptr(), 4, t["packed"].data_ptr(), 4,
+                                  t["r"].data_ptr(), t["cw"].data_ptr(), t["bias"].data_ptr(), 2, m, n, k, out.data_ptr(), 2,
+                                  ws_ptr, ws_bytes, None)
+        torch.cuda.synchronize()
+        assert rc == 0
+        return out.clone()
+    assert torch.equal(call(None, 0), single)
+    assert torch.equal(call(ws.data_ptr(), need - 1), single)        # too small: not used
+    assert torch.equal(call(ws.data_ptr(), need), split)
+    assert lib.oq_packed_linear_workspace_bytes(16, n, k, 4, 1, 4) == 0   # the streaming kernel needs none
+
+    # float activations: the operand-order copy lives in the workspace; without one, the LDS-staged kernel, same sums
+    m2, n2, k2 = 520, 200, 1152
+    layer2 = make_layer(rng, n2, k2, 3, 4)
+    x = torch.from_numpy(rng.standard_normal((m2, k2)).astype(F32)).to(torch.bfloat16).to(dev)
+    packed, r, cw = torch.from_numpy(layer2["packed"]).to(dev), layer2["r"].to(dev), torch.from_numpy(layer2["cw"]).to(dev)
+    want = ops.matmul_packed_weight_values(x, packed, r, cw, bits=3, out_features=n2, in_features=k2)
+    need2 = int(lib.oq_matmul_packed_weight_workspace_bytes(m2, n2, k2, 3, 2))
+    assert need2 == ((m2 + 31) // 32) * (k2 // 64) * 256 * 16
+    out2 = torch.empty(m2, n2, dtype=torch.bfloat16, device=dev)
+    ws2 = torch.empty(need2, dtype=torch.uint8, device=dev)
+    for ws_ptr, ws_bytes in ((None, 0), (ws2.data_ptr(), need2), (ws2.data_ptr(), 64)):
+        out2.zero_()
+        rc = lib.oq_matmul_packed_weight(x.data_ptr(), 2, None, packed.data_ptr(), 3, r.data_ptr(), cw.data_ptr(), None, 0,
+                                         m2, n2, k2, out2.data_ptr(), 2, ws_ptr, ws_bytes, None)
+        torch.cuda.synchronize()
+        assert rc == 0 and torch.equal(out2, want)
 
 
 def test_packed_linear_chooses_shared_k_for_short_and_long_problems(dev):
@@ -690,9 +746,9 @@ def test_matmul_packed_weight_large_m_bf16(dev, bits, m, n, k, library_switch):
 
 @pytest.mark.parametrize("bits,m", [(2, 520), (3, 520), (4, 520), (6, 520), (8, 520), (4, 3), (3, 40), (2, 130)])
 def test_matmul_packed_weight_large_m_bf16_under_graph_capture(dev, bits, m):
-    """While a stream is captured the float-activation call on bf16 values may not allocate: every wavefront
-    stages its own activation rows through LDS instead.  Same tile kernel, same sums: the replayed
-    graph returns the bits of the eager call, replay after replay."""
+    """The float-activation call on bf16 values under stream capture: the wrapper's workspace comes from the
+    graph's memory pool, the call takes the kernels the eager call takes, and the replayed graph returns
+    the bits of the eager call, replay after replay."""
     from orbitquant_amd import ops
 
     rng = np.random.default_rng(bits + m)

@@ -188,7 +188,7 @@ def test_value_outputs(dev, values):
         assert fast[0] is None and torch.equal(fast[1], plain[1]) and torch.equal(fast[2], plain[2])
 
 
-def test_plan_for_another_shape_writes_nothing(dev):
+def test_plan_for_another_shape_is_loud(dev):
     from orbitquant_amd import ops
 
     perm, signs, h, inv, cents, bounds, t = constants(dev, 1024, 256, 4)
@@ -205,7 +205,13 @@ def test_plan_for_another_shape_writes_nothing(dev):
                                 norms.data_ptr(), None)
     torch.cuda.synchronize()
     assert rc == 0
-    assert bool((lib_codes == 0xAB).all()) and bool((norms == -1.0).all())
+    # the kernel does not walk a plan built for another block size: no codes, and NaN norms, so that
+    # whatever is computed from this call's outputs is NaN instead of looking like a result
+    assert bool((lib_codes == 0xAB).all()) and bool(torch.isnan(norms).all())
+    # the Python wrapper knows what the plan was built for and refuses it before any launch
+    with pytest.raises(ValueError, match="rotate plan was built for"):
+        ops.rotate_quantize(x, t["perm"], t["signs"], t["bounds"], block_size=256, eps=1e-10, inv_sqrt_block=float(inv),
+                            code_format="u8", plan=wrong)
 
 
 def test_layer_uses_the_plan_and_matches_the_two_call_path(dev):

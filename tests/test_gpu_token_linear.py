@@ -122,7 +122,7 @@ def test_quantized_linear_argument_checks(dev):
             c["x"].data_ptr(), 2, None, m, 512, c["perm"].data_ptr(), c["signs"].data_ptr(), c["bounds"].data_ptr(),
             c["cents"].data_ptr(), a_bits, c["kw"]["block_size"], 1e-10, c["kw"]["inv_sqrt_block"], None,
             c["packed"].data_ptr(), 4, c["rn"].data_ptr(), c["wcents"].data_ptr(), None, 0, 256,
-            codes, norms, out.data_ptr(), 2, None, None)
+            codes, norms, out.data_ptr(), 2, None, None, 0, None)
 
     assert call(2, None, None) == 1 and b"scratch" in lib.oq_last_error()   # two tokens need the scratch buffers
     assert call(1, None, None) == 0                                           # one token does not
@@ -180,3 +180,34 @@ def test_shared_input_quantization(dev, m, monkeypatch):
     assert len(calls) == 4
     v(y)
     assert len(calls) == 5
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                                    # another stream: not served from the entry
+        before = len(calls)
+        on_side = v(y)
+        assert len(calls) == before + 1
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert torch.equal(on_side, v(y))
+
+
+def test_shared_input_quantization_under_inference_mode(dev, monkeypatch):
+    """Inference tensors have no version counter: such inputs are quantized by every layer (and the call
+    does not raise); outputs equal the plain forward."""
+    from orbitquant_amd import OrbitLinear, OrbitQuantConfig, layers as layers_mod, ops
+
+    torch.manual_seed(12)
+    cfg = OrbitQuantConfig(weight_bits=4, activation_bits=4)
+    q, k = (OrbitLinear.from_linear(torch.nn.Linear(1024, n), config=cfg).to(dev) for n in (512, 256))
+    calls = []
+    real = ops.rotate_quantize
+    monkeypatch.setattr(layers_mod.ops, "rotate_quantize", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    with torch.inference_mode():
+        x = torch.randn(8, 1024, device=dev, dtype=torch.bfloat16)
+        want = [layer(x) for layer in (q, k)]
+        for layer in (q, k):
+            layer.share_input_quantization = True
+        layers_mod._last_quantization.clear()
+        got = [layer(x) for layer in (q, k)]
+    assert len(calls) == 2
+    assert all(torch.equal(a, b) for a, b in zip(got, want))

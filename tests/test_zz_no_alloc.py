@@ -70,7 +70,7 @@ def call(layer, x, *, static):
         nibble = layer["abits"] <= 4 and k % 2 == 0
         codes = torch.empty((m, k // 2 if nibble else k), dtype=torch.uint8, device=x.device)
         norms = torch.empty(m, dtype=torch.float32, device=x.device)
-        rc = lib.oq_quantized_linear(*head, codes.data_ptr(), norms.data_ptr(), out.data_ptr(), dt, None, stream)
+        rc = lib.oq_quantized_linear(*head, codes.data_ptr(), norms.data_ptr(), out.data_ptr(), dt, None, None, 0, stream)
     torch.cuda.synchronize()
     return rc, out
 
