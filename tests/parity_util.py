@@ -47,6 +47,27 @@ def output_error(got, want, s, r, k, out_is_16bit: bool, out_is_bf16: bool = Tru
     return strict, rounded
 
 
+def outside_rounded_bound(got, want, s, r, k, out_is_bf16: bool = True) -> int:
+    """For a 16-bit output: the number of elements that are NOT the rounding of any value within the stated
+    bound of `want`.  Rounding to the output format is monotonic, so that is
+        round(want - bound) <= got <= round(want + bound)
+    element by element.  Zero means: wherever a stored output exceeds the bound, the excess is the rounding
+    of the stored 16-bit value and nothing else - the kernel's result before that rounding may have met it."""
+    import torch
+
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    bound = 2e-2 * np.asarray(s, np.float64)[:, None] * np.asarray(r, np.float64)[None, :] / math.sqrt(k)
+    dtype = torch.bfloat16 if out_is_bf16 else torch.float16
+
+    def rounded(a):
+        return torch.from_numpy(a).to(torch.float32).to(dtype).double().numpy()
+    # (the fp64 -> fp32 step before the 16-bit rounding is widened by one fp32 spacing: it must not tighten the interval)
+    lo = rounded(np.nextafter((want - bound).astype(np.float32), np.float32(-np.inf)).astype(np.float64))
+    hi = rounded(np.nextafter((want + bound).astype(np.float32), np.float32(np.inf)).astype(np.float64))
+    return int(((got < lo) | (got > hi)).sum())
+
+
 def cosine(got, want) -> float:
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)

@@ -265,3 +265,126 @@ def test_adaln_module_survives_dtype_casts_of_the_model():
         assert layer.scales.dtype == torch.bfloat16 and torch.equal(layer.scales, scales)
         assert layer.packed_weight.dtype == torch.uint8 and torch.equal(layer.packed_weight, packed)
     assert model[0].weight.dtype == torch.bfloat16 and layer.bias.dtype == torch.bfloat16
+
+
+# ------------------------------------------------- an artifact the REFERENCE wrote (tests/golden/artifact_tiny)
+
+GOLDEN_ARTIFACT = __import__("pathlib").Path(__file__).resolve().parent / "golden" / "artifact_tiny"
+
+
+class FluxTransformer2DModel(torch.nn.Module):
+    """The architecture tests/golden/make_artifact_golden.py quantized with the reference (same module names)."""
+
+    def __init__(self, dim=64):
+        super().__init__()
+
+        def block():
+            return torch.nn.ModuleDict({
+                "norm1": torch.nn.ModuleDict({"linear": torch.nn.Linear(dim, 6 * dim)}),
+                "attn": torch.nn.ModuleDict({"to_q": torch.nn.Linear(dim, dim), "to_k": torch.nn.Linear(dim, dim),
+                                             "to_v": torch.nn.Linear(dim, dim, bias=False),
+                                             "to_out": torch.nn.ModuleList([torch.nn.Linear(dim, dim)])}),
+                "ff": torch.nn.ModuleDict({"net": torch.nn.ModuleList([
+                    torch.nn.ModuleDict({"proj": torch.nn.Linear(dim, 2 * dim)}), torch.nn.Identity(),
+                    torch.nn.Linear(2 * dim, dim)])}),
+            })
+        self.transformer_blocks = torch.nn.ModuleList([block() for _ in range(3)])
+        self.proj_out = torch.nn.Linear(dim, dim)
+
+
+def golden_artifact_oracle_outputs(name, x32):
+    """fp64 output of quantized module `name` of the golden artifact on fp32 rows x32, computed by the oracle
+    from the artifact's OWN files (state tensors, codebook and rotation sidecars, config, manifest):
+    -> (want, token norms, row norms) for an OrbitLinear, (want, None, None) for an AdaLN module."""
+    from safetensors.torch import load_file
+
+    from oracle import oracle_c
+
+    manifest = json.loads((GOLDEN_ARTIFACT / "orbitquant_manifest.json").read_text())
+    config = json.loads((GOLDEN_ARTIFACT / "quantization_config.json").read_text())
+    state = load_file(GOLDEN_ARTIFACT / "model.safetensors")
+    bias = state.get(name + ".bias")
+    bias = None if bias is None else bias.float().numpy()
+    if name in manifest["adaln_modules"]:
+        scales = state[name + ".scales"].float().numpy()
+        n, groups = scales.shape
+        g = int(config["adaln_group_size"])
+        packed = state[name + ".packed_weight"].numpy()
+        codes = np.stack([packed & 15, packed >> 4], axis=-1).reshape(n, groups * g)
+        return o.adaln_linear_f64(x32, codes, scales, bias, x32.shape[1], g), None, None
+    books = load_file(GOLDEN_ARTIFACT / "orbitquant_codebooks.safetensors")
+    rots = load_file(GOLDEN_ARTIFACT / "orbitquant_rotations.safetensors")
+    k = x32.shape[1]
+    w_bits = int(manifest.get("module_bits", {}).get(name, manifest["weight_bits"]))
+    a_bits = int(manifest["activation_bits"])
+    rot = f"dim{k}_seed{config['rotation_seed']}_block{config['block_size']}"
+    perm, signs = rots[rot + ".permutation"].numpy(), rots[rot + ".signs"].numpy()
+    inv = np.float32(rots[rot + ".normalization"].reshape(-1)[0].item())
+    ca, ba = books[f"dim{k}_bits{a_bits}.centroids"].numpy(), books[f"dim{k}_bits{a_bits}.boundaries"].numpy()
+    cw = books[f"dim{k}_bits{w_bits}.centroids"].numpy()
+    codes, s = oracle_c.rotate_quantize(x32, perm, signs, ba, int(config["block_size"]), float(config["activation_eps"]), inv)
+    r = state[name + ".row_norms"].float().numpy()
+    want = oracle_c.linear_from_codes(codes, s, ca, state[name + ".packed_weight_indices"].numpy(), w_bits, r, cw, bias, r.size)
+    return want, s, r
+
+
+def test_reference_written_artifact_loads_strictly():
+    """The artifact directory was written by the reference's own save_orbitquant_artifact (a mixed-bit model:
+    2-bit weights, first and last block protected at 4 bits, three AdaLN modules): this package's loader takes
+    it as it is - checksums, sidecars equal to this package's generators, strict state dict."""
+    import re
+
+    from safetensors.torch import load_file
+
+    from orbitquant_amd import OrbitLinear, RTNInt4Linear, load_artifact
+
+    model = FluxTransformer2DModel()
+    manifest = load_artifact(model, GOLDEN_ARTIFACT)
+    assert manifest["artifact_format"] == "orbitquant-v1" and len(manifest["quantized_modules"]) == 18
+    state = load_file(GOLDEN_ARTIFACT / "model.safetensors")
+    got = model.state_dict()
+    assert set(got) == set(state)
+    for key, value in state.items():
+        assert torch.equal(got[key].cpu(), value), key
+    for name in manifest["quantized_modules"]:
+        layer = dict(model.named_modules())[name]
+        bits = manifest["module_bits"].get(name, 2)
+        assert isinstance(layer, OrbitLinear) and layer.weight_bits == bits and layer.activation_bits == 4
+        assert layer.rotation.block_size == 16
+        assert state[name + ".packed_weight_indices"].numel() == layer.out_features * layer.in_features * bits // 8
+        assert state[name + ".row_norms"].dtype == torch.bfloat16
+    assert {manifest["module_bits"][n] for n in manifest["module_bits"]} == {4}
+    assert sum(1 for n in manifest["quantized_modules"] if n not in manifest["module_bits"]) == 6   # the middle block: 2 bits
+    for name in manifest["adaln_modules"]:
+        assert isinstance(dict(model.named_modules())[name], RTNInt4Linear)
+    assert isinstance(model.proj_out, torch.nn.Linear)   # skipped by the reference's policy: left alone
+    # sidecar key names are what the reference's validator accepts (src/orbitquant/artifacts/validator.py:32-38)
+    for key in load_file(GOLDEN_ARTIFACT / "orbitquant_codebooks.safetensors"):
+        assert re.fullmatch(r"dim\d+_bits\d+\.(centroids|boundaries)", key), key
+    for key in load_file(GOLDEN_ARTIFACT / "orbitquant_rotations.safetensors"):
+        assert re.fullmatch(r"dim\d+_seed\d+_block\d+\.(permutation|inverse_permutation|signs|normalization)", key), key
+
+
+def test_oracle_reads_the_reference_artifact_like_the_reference_does():
+    """What the artifact's tensors MEAN: the oracle, fed only from the artifact's files, reproduces the outputs the
+    reference's own modules gave on the same inputs (its CPU dequant_bf16 forward, stored beside the artifact)
+    within the error bound of the path - so the loader's reading of the layout is pinned by the reference, not
+    by this package's writer."""
+    from safetensors.torch import load_file
+
+    outputs = load_file(GOLDEN_ARTIFACT / "reference_outputs.safetensors")
+    record = json.loads((GOLDEN_ARTIFACT / "reference_outputs.json").read_text())
+    assert len(record["modules"]) == 21
+    for name, kind in record["modules"].items():
+        x, y = outputs[name + ".x"].numpy(), outputs[name + ".y"].numpy().astype(np.float64)
+        want, s, r = golden_artifact_oracle_outputs(name, x)
+        if kind == "RTNInt4Linear":
+            # the reference's module rounds its output to bf16 (and accumulates in bf16-sized steps on some back-ends)
+            assert np.abs(y - want).max() <= 2.0 ** -7 * np.abs(want).max(), name
+            continue
+        k = x.shape[1]
+        bound = 2e-2 * s[:, None].astype(np.float64) * r[None, :] / np.sqrt(k)
+        err = np.abs(y - want)
+        assert (err <= bound + 1e-6).all(), (name, float((err / (bound + 1e-30)).max()))
+        assert float((y * want).sum() / (np.linalg.norm(y) * np.linalg.norm(want))) >= 0.9999, name
+        assert np.array_equal(y[2], want[2])   # the zero token: exactly the bias

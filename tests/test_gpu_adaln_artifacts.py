@@ -126,3 +126,65 @@ def test_gpu_adaln_weight_quantizer_equals_the_oracle(N, K, group, dtype):
     want_packed, want_scales, _ = o.adaln_quantize(w.float().numpy(), group)
     assert np.array_equal(scales.cpu().numpy(), want_scales)
     assert np.array_equal(packed.cpu().numpy(), want_packed)
+
+
+def test_layers_restored_from_the_reference_written_artifact_match_the_oracle():
+    """tests/golden/artifact_tiny was written by the reference's save_orbitquant_artifact.  Loaded by this
+    package's loader onto the GPU, every restored OrbitLinear gives, on the inputs stored beside the artifact,
+    the oracle's result computed from the artifact's own files (codes of the restored layer's quantizer bit for
+    bit, outputs within the error bound) - and with that the reference's own outputs; the AdaLN modules match
+    their fp64 contract within the bf16 rounding of the output."""
+    from safetensors.torch import load_file
+
+    from orbitquant_amd import OrbitLinear, load_artifact, ops
+    from oracle import oracle_c
+    from test_adaln_and_artifacts import GOLDEN_ARTIFACT, FluxTransformer2DModel, golden_artifact_oracle_outputs
+
+    dev = torch.device("cuda:0")
+    model = FluxTransformer2DModel()
+    manifest = load_artifact(model, GOLDEN_ARTIFACT, device=dev)
+    modules = dict(model.named_modules())
+    outputs = load_file(GOLDEN_ARTIFACT / "reference_outputs.safetensors")
+    rots = load_file(GOLDEN_ARTIFACT / "orbitquant_rotations.safetensors")
+    books = load_file(GOLDEN_ARTIFACT / "orbitquant_codebooks.safetensors")
+    for name in manifest["quantized_modules"]:
+        layer = modules[name]
+        assert isinstance(layer, OrbitLinear) and layer.packed_weight_indices.device.type == "cuda"
+        x = outputs[name + ".x"]
+        y_ref = outputs[name + ".y"].numpy().astype(np.float64)
+        want, s, r = golden_artifact_oracle_outputs(name, x.numpy())
+        k = x.shape[1]
+        # the restored layer's quantizer against the oracle on the artifact's sidecar tables: bit for bit
+        perm = rots[f"dim{k}_seed0_block16.permutation"].numpy()
+        signs = rots[f"dim{k}_seed0_block16.signs"].numpy()
+        inv = np.float32(rots[f"dim{k}_seed0_block16.normalization"].reshape(-1)[0].item())
+        want_codes, want_s = oracle_c.rotate_quantize(x.numpy(), perm, signs, books[f"dim{k}_bits4.boundaries"].numpy(), 16, 1e-10, inv)
+        codes, _, norms = ops.rotate_quantize(x.to(dev), layer._rotation_permutation, layer._rotation_signs,
+                                              layer._activation_codebook_boundaries, block_size=layer.rotation.block_size,
+                                              eps=layer.activation_eps, inv_sqrt_block=layer.rotation.normalization, code_format="u8")
+        assert np.array_equal(codes.cpu().numpy(), want_codes), name
+        assert np.array_equal(norms.cpu().numpy().view(np.int32), want_s.view(np.int32)), name
+        bound = 2e-2 * s[:, None].astype(np.float64) * r[None, :] / np.sqrt(k)
+        got = layer(x.to(dev)).double().cpu().numpy()                 # fp32 in, fp32 out
+        assert (np.abs(got - want) <= bound + 1e-7).all(), name
+        assert float((got * want).sum() / (np.linalg.norm(got) * np.linalg.norm(want))) >= 0.9999, name
+        assert (np.abs(got - y_ref) <= bound + 1e-6).all(), name       # ... and the reference's own module output
+        got16 = layer(x.to(dev).to(torch.bfloat16))
+        want16, s16, _ = golden_artifact_oracle_outputs(name, x.to(torch.bfloat16).float().numpy())
+        bound16 = 2e-2 * s16[:, None].astype(np.float64) * r[None, :] / np.sqrt(k)
+        err16 = np.abs(got16.double().cpu().numpy() - want16)
+        assert (err16 <= bound16 + np.abs(want16) * 2.0 ** -8 + 1e-7).all(), name
+    for name in manifest["adaln_modules"]:
+        x = outputs[name + ".x"]                                        # bf16-representable
+        want, _, _ = golden_artifact_oracle_outputs(name, x.numpy())
+        got = modules[name](x.to(dev)).double().cpu().numpy()
+        # fp32 accumulation of exact bf16 products, then one rounding to bf16 (the bound of the AdaLN kernel's own test)
+        k = x.shape[1]
+        zero, _, _ = golden_artifact_oracle_outputs(name, np.zeros((1, k), np.float32))           # the bias
+        weights, _, _ = golden_artifact_oracle_outputs(name, np.eye(k, dtype=np.float32))          # rows: W[:, j] + bias
+        mass = np.abs(x.numpy().astype(np.float64)) @ np.abs(weights - zero) + np.abs(zero)
+        # (the artifact holds an fp32 bias; the packed AdaLN kernel takes it as bf16, like the reference's kernels for it)
+        tolerance = np.abs(want) * 2.0 ** -8 + np.abs(zero) * 2.0 ** -8 + mass * k * 2.0 ** -24 + 1e-30
+        assert (np.abs(got - want) <= tolerance).all(), (name, float((np.abs(got - want) / tolerance).max()))
+        y_ref = outputs[name + ".y"].numpy().astype(np.float64)
+        assert np.abs(got - y_ref).max() <= 2.0 ** -7 * np.abs(want).max(), name

@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from oracle import oracle_c, oracle_np as o
-from parity_util import cosine, output_error, reference_tables
+from parity_util import cosine, output_error, outside_rounded_bound, reference_tables
 
 pytestmark = pytest.mark.gpu
 
@@ -98,5 +98,8 @@ def test_full_size_layer(dev, name, m, k, n, wbits, abits, kind):
     got = out[rows].float().cpu().numpy()
     strict, rounded = output_error(got, want, want_s[rows], r.float().numpy(), k, True, True)
     assert rounded <= 1.0, f"{name}: max error is {rounded:.3f} of the bound ({strict:.3f} without bf16's half-ulp)"
+    # every stored output is the rounding of a value within the stated bound: any excess is the bf16 rounding alone
+    bad = outside_rounded_bound(got, want, want_s[rows], r.float().numpy(), k, True)
+    assert bad == 0, f"{name}: {bad} outputs are not the rounding of any value within the bound"
     cos = cosine(got, want)
     assert cos >= 0.9999, f"{name}: cosine {cos}"

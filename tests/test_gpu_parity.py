@@ -14,7 +14,7 @@ import pytest
 import torch
 
 from oracle import oracle_c, oracle_np as o
-from parity_util import cosine, output_error, reference_tables
+from parity_util import cosine, output_error, outside_rounded_bound, reference_tables
 
 pytestmark = pytest.mark.gpu
 
@@ -229,6 +229,9 @@ def check_outputs(got, want, s, r, k, what=""):
     is16 = out_dtype != torch.float32
     strict, rounded = output_error(got, want, s, r, k, is16, out_dtype == torch.bfloat16)
     assert rounded <= 1.0, f"{what}: max error is {rounded:.3f} of the bound ({strict:.3f} without the output format's half-ulp)"
+    if is16:   # every stored output must be the rounding of a value within the stated bound: any excess is output rounding alone
+        bad = outside_rounded_bound(got, want, s, r, k, out_dtype == torch.bfloat16)
+        assert bad == 0, f"{what}: {bad} outputs are not the rounding of any value within the bound"
     cos = cosine(got, want)
     assert cos >= 0.9999, f"{what}: cosine {cos}"
     return rounded, cos
