@@ -574,6 +574,58 @@ def c3_gemm_lines(device, iters):
     return out
 
 
+def c4_gemm_lines(device, iters):
+    """The two packed GEMMs of the video-DiT FFN (c4: W4A6, M = 32760, one activation code per byte), each
+    timed alone: the largest configuration, on the byte-code form of the tile kernel."""
+    spec = workload_spec("c4", 0)
+    gen = torch.Generator().manual_seed(4)
+    layers = build_layers(spec, device, gen, False, activation="separate")
+    out = {}
+    for layer, _act in layers:
+        k, n = layer.in_features, layer.out_features
+        x = make_input(spec, k, gen).to(device)
+        t = time_kernel(gemm_only_closure(layer, x), max(3, iters // 10))
+        tflops = 2.0 * spec["M"] * n * k / t / 1e12
+        out[f"{k}->{n}"] = {"gemm_us": t * 1e6, "gemm_tflops": tflops, "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "codes": "one 6-bit code per byte"}
+        del x
+    torch.cuda.empty_cache()
+    return out
+
+
+def adaln_lines(device, iters):
+    """The AdaLN INT4 group-64 linear (the other quantized linear of a DiT block) at the DiT-XL/2 modulation
+    shape, 1152 -> 6912, one and sixteen tokens: microseconds per launch and GB/s of packed bytes (indices +
+    bf16 scales) against HBM.  The matrix is 4.1 MB: the figure is about launch and latency, not streaming."""
+    from orbitquant_amd import _lib, ops
+
+    lib = _lib.load()
+    k, n, g = 1152, 6912, 64
+    gen = torch.Generator().manual_seed(7)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(device)
+    packed, scales = ops.quantize_adaln_weight(w, group_size=g)
+    scales = scales.to(torch.bfloat16)
+    bias = torch.zeros(n, dtype=torch.bfloat16, device=device)
+    nbytes = packed.numel() + 2 * scales.numel()
+    out = {}
+    for m in (1, 16):
+        x = torch.randn(m, k, generator=gen).to(torch.bfloat16).to(device)
+        y = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+        want = ops.adaln_int4_linear(x, packed, scales, out_features=n, in_features=k, group_size=g, bias=bias)
+        args = (x.data_ptr(), packed.data_ptr(), scales.data_ptr(), bias.data_ptr(), m, n, k, g, y.data_ptr())
+
+        def fn():
+            if lib.oq_matmul_packed_adaln_int4(*args, torch.cuda.current_stream().cuda_stream) != 0:
+                raise RuntimeError(lib.oq_last_error().decode())
+        fn()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+        t = time_kernel(fn, max(10, iters))
+        out[f"M={m}"] = {"launch_us": t * 1e6, "gbs": nbytes / t / 1e9, "frac_of_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS}
+    out["shape"] = [n, k]
+    out["packed_bytes"] = nbytes
+    return out
+
+
 def float_activation_lines(device, iters):
     """`oq_matmul_packed_weight` (bf16 activation values times the packed weight, the reference's generic
     contract) on the two c2 shapes: the whole call, i.e. the pass that puts the activations into operand
@@ -860,6 +912,8 @@ def main() -> int:
         out["roofline_small_m"] = small_m_roofline(device, args.kernel_iters)
         out["c3_gemms"] = c3_gemm_lines(device, args.kernel_iters)
         out["float_activations"] = float_activation_lines(device, args.kernel_iters)
+        out["c4_gemms"] = c4_gemm_lines(device, args.kernel_iters)
+        out["adaln"] = adaln_lines(device, args.kernel_iters)
         out["decode_stack"] = measure_c5(args, device, brief=True)
     copy_calibration(device)
     if not args.no_cpu_baseline:
