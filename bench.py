@@ -259,6 +259,41 @@ def _code_format(layer, x):
     return "u8" if (tokens > 16 and k % 64 == 0) or k % 128 == 0 else None
 
 
+def chunked_step_closure(layers, x, chunks, streams=2):
+    """The step in `chunks` row chunks dealt round `streams` ordinary (equal-priority) streams, each chunk its own
+    chain of oq_quantized_linear calls (rows are independent): the quantizer of one chunk runs beside the matmul
+    of another, on the CUs a 192-workgroup matmul leaves idle.  Host-side ordering only (events); None when
+    the step has no bare-call form.  Returns (step, outputs) with outputs the list of per-chunk output tensors."""
+    m = x.shape[0]
+    if m % chunks != 0:
+        return None
+    rows = m // chunks
+    chains = []
+    for c in range(chunks):
+        raws, h = [], x[c * rows:(c + 1) * rows]
+        for i, (layer, act) in enumerate(layers):
+            if _code_format(layer, h) is None or act == "slice3072" or (act == "gelu" and not activation_is_fused(layers, i)):
+                return None
+            raw = RawLinear(layer, h)
+            raws.append(raw)
+            h = raw.out
+        chains.append(raws)
+    side = [torch.cuda.Stream() for _ in range(streams)]
+
+    def step():
+        main = torch.cuda.current_stream()
+        for st in side:
+            st.wait_stream(main)
+        for c, raws in enumerate(chains):
+            with torch.cuda.stream(side[c % streams]):
+                for raw in raws:
+                    raw.linear()
+        for st in side:
+            main.wait_stream(st)
+        return [raws[-1].out for raws in chains]
+    return step
+
+
 class RawLinear:
     """One OrbitLinear as bare C-ABI calls into buffers allocated once: what a native host does.
 
@@ -861,6 +896,40 @@ def main() -> int:
         abi_dt = time_steps(abi, args.steps, args.warmup)
         if abi_dt < dt:
             dt, launch = abi_dt, "c_abi"
+    # the same calls in row chunks on two streams (quantizer of one chunk beside the matmul of another)
+    chunked = {}
+    if abi is not None and args.workload == "c2":
+        want = run_step(layers, x)
+        for chunks in (2, 4):
+            step = chunked_step_closure(layers, x, chunks)
+            if step is None:
+                continue
+            got = torch.cat(step(), dim=0)
+            torch.cuda.synchronize()
+            same = torch.equal(got, want)
+            close = same or bool((got.float() - want.float()).abs().max() <= want.float().abs().max() * 2.0 ** -7)
+            if not close:
+                raise AssertionError("the chunked step differs from the module step")
+            cdt = time_steps(step, args.steps, args.warmup)
+            chunked[f"{chunks}_chunks_2_streams_ms"] = cdt * 1e3
+            chunked[f"{chunks}_chunks_bit_identical"] = same
+            if not args.no_graph:   # the same fork and join as one HIP graph (branches of a graph need no host-side events)
+                try:
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        outs = step()
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    if torch.equal(torch.cat(outs, dim=0), got):
+                        gdt = time_steps(graph.replay, args.steps, args.warmup)
+                        chunked[f"{chunks}_chunks_2_streams_graph_ms"] = gdt * 1e3
+                        if same and gdt < dt:
+                            dt, launch = gdt, f"hipgraph, {chunks} row chunks on 2 streams"
+                except Exception as exc:
+                    chunked[f"{chunks}_chunks_graph_error"] = str(exc)[:200]
+            if same and cdt < dt:
+                dt, launch = cdt, f"c_abi, {chunks} row chunks on 2 streams"
 
     # dominant kernel alone: the packed GEMM of the first layer, and every other piece for the record
     pieces = {}
@@ -891,6 +960,7 @@ def main() -> int:
                    "flop_per_step": flops, "launch": launch, "eager_ms_per_step": eager_dt * 1e3,
                    "graph_ms_per_step": None if graph_dt is None else graph_dt * 1e3,
                    "c_abi_ms_per_step": None if abi_dt is None else abi_dt * 1e3,
+                   "row_chunks_on_two_streams": chunked,
                    "preroll_s": PREROLL_SECONDS,
                    "activation": ("gelu as a 65536-entry table of torch's own results, looked up in the producing "
                                   "matmul's epilogue" if any(l._output_activation_table is not None for l, _ in layers)
