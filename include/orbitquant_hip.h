@@ -162,6 +162,9 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
  * tests and measurements that compare variants inside one process change a switch through this
  * call.  Results stay correct under every setting; only which kernel computes them changes.
  * Not thread-safe against running calls.  No counterpart in the reference.
+ * Refused (OQ_ERR_INVALID) unless the process was started with ORBITQUANT_DEBUG=1 in its
+ * environment: a serving process cannot have its kernels, and so the bits of its results,
+ * switched under it.
  */
 int oq_debug_override(const char *name, const char *value);
 

@@ -54,10 +54,13 @@ const char *const kEnvNames[ENV_COUNT] = {"OQ_GEMM_TILE", "OQ_NO_TOKEN_LINEAR", 
                                           "OQ_RQ_FAST_MIN_M", "OQ_NO_GEMV_GROUP", "OQ_GEMV_GROUP_R", "OQ_GEMV_NO_ASTAGE",
                                           "OQ_GEMV_MAX_M", "OQ_GEMM_WG_SPLIT", "OQ_FLOAT_GEMM_MIN_M", "OQ_GEMM_STAMPS"};
 const char *env_values[ENV_COUNT];
+bool overrides_allowed = false;  // ORBITQUANT_DEBUG=1 in the environment the process started with
 void env_load() {
   static std::once_flag once;
   std::call_once(once, [] {
     for (int i = 0; i < ENV_COUNT; ++i) env_values[i] = getenv(kEnvNames[i]);
+    const char *debug = getenv("ORBITQUANT_DEBUG");
+    overrides_allowed = debug != nullptr && strcmp(debug, "1") == 0;
   });
 }
 }  // namespace
@@ -71,6 +74,8 @@ const char *debug_env(int which) {
 
 int debug_env_set(const char *name, const char *value) {
   env_load();
+  if (!overrides_allowed)  // a switch changes which kernel runs and so the bits of a result: not for a serving process
+    return fail(OQ_ERR_INVALID, "debug_override: switches are fixed in this process (start it with ORBITQUANT_DEBUG=1 to change them at run time)");
   for (int i = 0; i < ENV_COUNT; ++i) {
     if (strcmp(name, kEnvNames[i]) == 0) {
       env_values[i] = value != nullptr ? strdup(value) : nullptr;  // a few bytes per call, never freed: readers may hold the old one

@@ -291,10 +291,14 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
               }
             }
           }
+#ifdef OQ_RQ_TIMING_NO_SUMSQ  // timing experiment only: what the pass would cost if the sums came from elsewhere
+          q = q + f[0];
+#else
           float sq[kChunk];
 #pragma unroll
           for (int e = 0; e < kChunk; ++e) sq[e] = f[e] * f[e];
           q = q + (((sq[0] + sq[1]) + (sq[2] + sq[3])) + ((sq[4] + sq[5]) + (sq[6] + sq[7])));
+#endif
         }
         if (pb + kBatch < a.passes) request(b, pb + b + kBatch);  // refill the slot: four passes stay in flight
       }

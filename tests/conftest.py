@@ -10,6 +10,10 @@ if str(ROOT) not in sys.path:
 
 GOLDEN = Path(__file__).resolve().parent / "golden"
 
+# lets the tests switch kernel variants inside the process (oq_debug_override refuses without it);
+# the library reads it at its first call, so it has to be there before any test loads the library
+os.environ.setdefault("ORBITQUANT_DEBUG", "1")
+
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")

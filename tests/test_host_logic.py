@@ -45,6 +45,23 @@ def test_debug_override_knows_its_switches():
     assert lib.oq_debug_override(None, b"1") != 0
 
 
+def test_debug_override_is_refused_in_a_process_started_without_the_debug_variable():
+    """A serving process cannot have its kernel variants switched at run time: without ORBITQUANT_DEBUG=1
+    in its starting environment the call fails and says why."""
+    import os
+    import subprocess
+    import sys
+
+    code = ("from orbitquant_amd import _lib; lib = _lib.load(); rc = lib.oq_debug_override(b'OQ_GEMM_TILE', b'3'); "
+            "print(rc, lib.oq_last_error().decode())")
+    env = {k: v for k, v in os.environ.items() if k != "ORBITQUANT_DEBUG"}
+    root = str(Path(__file__).resolve().parent.parent)
+    done = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stderr
+    rc, message = done.stdout.strip().split(" ", 1)
+    assert int(rc) != 0 and "ORBITQUANT_DEBUG=1" in message
+
+
 def test_product_codebooks_match_reference_generated_fixture(golden_dir):
     from orbitquant_amd.codebooks import get_codebook
 
