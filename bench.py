@@ -41,6 +41,10 @@ def parse_args():
                     help="c5: q, k and v each quantize their (common) input, as the reference's layers do")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP-graph replays")
     ap.add_argument("--kernel-iters", type=int, default=50)
+    ap.add_argument("--gemm-phases", action="store_true",
+                    help="print where the time inside one packed-GEMM launch of the workload goes (in-kernel clock stamps); "
+                         "needs a library built with -DOQ_GEMM_STAMPS: python -m orbitquant_amd.build --variant stamps "
+                         "--flags=-DOQ_GEMM_STAMPS --only packed_gemm.hip, then ORBITQUANT_HIP_LIB=orbitquant_amd/liborbitquant_hip_stamps.so")
     ap.add_argument("--activation", default="output", choices=["output", "input", "separate"],
                     help="where the GELU between two linears runs: as a table lookup in the epilogue of the "
                          "matmul that produces its input (default), in the quantize kernel of the layer that "
@@ -852,10 +856,70 @@ def bench_c5(args, device):
     print(json.dumps(out))
 
 
+# ------------------------------------------------------- inside one GEMM launch
+
+def gemm_phases(layers, x, launches=20):
+    """Text report of one packed-GEMM launch per layer of the step, from stamps every wavefront of the tile
+    kernel takes of the shader clock (s_memtime) and of the 100 MHz wall clock (s_memrealtime) as it passes:
+    first instruction, lookup tables written, loop entered, loop left, barrier passed, last store issued, done.
+    The stamps exist only in a library compiled with -DOQ_GEMM_STAMPS (a product build takes none)."""
+    from orbitquant_amd import _lib
+
+    lib = _lib.load()
+    dev = x.device
+    stamps = torch.zeros(8192 * 4 * 16, dtype=torch.int64, device=dev)
+
+    def switch(value):
+        if lib.oq_debug_override(b"OQ_GEMM_STAMPS", None if value is None else str(value).encode()) != 0:
+            raise RuntimeError(lib.oq_last_error().decode())
+
+    h = x
+    for i, (layer, act) in enumerate(layers):
+        raw = RawLinear(layer, h)
+        raw.quantize()
+        switch(None)
+        per_launch = time_kernel(raw.gemm, 50)
+        stamps.zero_()
+        switch(stamps.data_ptr())
+        for _ in range(launches):
+            raw.gemm()
+        torch.cuda.synchronize()
+        switch(None)
+        s = stamps.cpu().numpy().reshape(-1, 16)
+        s = s[s[:, 0] != 0]
+        if len(s) == 0:
+            raise SystemExit("no stamps were written: load a library built with -DOQ_GEMM_STAMPS (see --help)")
+        cycles = (s[:, 8] - s[:, 0]).astype(np.float64)
+        wall = (s[:, 7] - s[:, 6]).astype(np.float64)            # 10 ns ticks
+        mhz = cycles.sum() / wall.sum() * 100.0
+        fused = "+gelu" if activation_is_fused(layers, i) and act == "gelu" else ""
+        print(f"--- layer {i}{fused}: M={raw.m} N={raw.n} K={raw.k}, {len(s)} wavefronts stamped (the last of {launches} launches each), "
+              f"{per_launch * 1e6:.2f} us per launch by events (launch to launch), "
+              f"{(s[:, 7].max() - s[:, 6].min()) / 100.0:.2f} us first wavefront start to last wavefront end, shader clock {mhz:.0f} MHz")
+        skew = (s[:, 6] - s[:, 6].min()) / 100.0
+        print(f"    wavefront start after the first: median {np.median(skew):.2f}, max {skew.max():.2f} us; "
+              f"wavefront lifetime: median {np.median(wall) / 100:.2f}, max {wall.max() / 100:.2f} us")
+        rows = [("start -> kernel arguments read", 0, 10), ("-> centroids requested, tile mapped", 10, 13), ("-> operand addresses", 13, 14), ("-> first packed operands requested", 14, 15),
+                ("-> output-map window requested", 15, 11), ("-> centroids arrived", 11, 12),
+                ("-> lookup tables written", 12, 1), ("-> barrier, first lookups (loop entered)", 1, 2), ("main loop", 2, 3),
+                ("wait at the barrier after the loop", 3, 4), ("epilogue until the last store is issued", 4, 5), ("stores drained", 5, 8)]
+        for name, a, b in rows:
+            d = (s[:, b] - s[:, a]).astype(np.float64) / mhz
+            print(f"    {name:42s} median {np.median(d):6.2f}   p10 {np.percentile(d, 10):6.2f}   p90 {np.percentile(d, 90):6.2f}   max {d.max():6.2f} us")
+        steps = raw.k // 64
+        loop = (s[:, 3] - s[:, 2]).astype(np.float64)
+        print(f"    main loop: {np.median(loop) / steps:.0f} shader cycles per K-step of 64 (median over wavefronts; K-steps per wavefront when K is not shared: {steps})")
+        xcc = ((s[:, 9] >> 32) & 0xf).astype(np.int64)
+        print("    wavefronts per XCC:", np.bincount(xcc, minlength=8).tolist())
+        h = raw.out
+
+
 # ------------------------------------------------------------------------ main
 
 def main() -> int:
     args = parse_args()
+    if args.gemm_phases:
+        os.environ["ORBITQUANT_DEBUG"] = "1"   # the stamp buffer's address reaches the library through oq_debug_override
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
@@ -876,6 +940,9 @@ def main() -> int:
     flops = sum(2.0 * spec["M"] * n * k for (k, n, *_rest) in spec["layers"])
 
     preroll(lambda: run_step(layers, x))
+    if args.gemm_phases:
+        gemm_phases(layers, x)
+        return 0
     eager_dt = time_steps(lambda: run_step(layers, x), args.steps, args.warmup)
     dt, launch, graph_dt = eager_dt, "eager", None
     captured = None if args.no_graph else capture_step(lambda: run_step(layers, x))

@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, grp = lane >> 5;
 #ifdef OQ_GEMM_STAMPS
-  uint64_t stamp[8], stamp_extra[4] = {0, 0, 0, 0};
+  uint64_t stamp[8], stamp_extra[6] = {0, 0, 0, 0, 0, 0};
   stamp[0] = __builtin_amdgcn_s_memtime();
   stamp[6] = __builtin_amdgcn_s_memrealtime();
 #define OQ_STAMP(i) stamp[i] = __builtin_amdgcn_s_memtime()
@@ -169,9 +169,16 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
   const int group = bid / width;
   const int first_m = group * GROUP_M;
   const int gsz = min(g.tiles_m - first_m, GROUP_M);
-  const int pid_m = first_m + (bid % width) % gsz;
-  const int pid_n = (bid % width) / gsz;
+  const int in_group = bid - group * width;
+  // (full groups, the usual case, by shifts: a division by a run-time value is some thirty instructions)
+  const int pid_m = first_m + (gsz == GROUP_M ? in_group & (GROUP_M - 1) : in_group % gsz);
+  const int pid_n = gsz == GROUP_M ? in_group >> 2 : in_group / gsz;
+  static_assert(GROUP_M == 4);
 
+#ifdef OQ_GEMM_STAMPS
+  __asm__ volatile("" ::"s"(pid_n), "s"(pid_m));
+  stamp_extra[3] = __builtin_amdgcn_s_memtime();  // centroids requested, tile mapped
+#endif
   const uint32_t lds_base = lds_byte_address(lds);           // a multiple of 65536 by the alignment
   const uint32_t w_off = lds_base + 4 * r, a_off = lds_base + 128 + 4 * r;  // the lane's copy inside a table row
   const int wm = KSPLIT == 1 ? (wave >> 1) * (FM * 32) : 0, wn = KSPLIT == 1 ? (wave & 1) * (FN * 32) : 0;
@@ -189,6 +196,14 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
   uint32_t a_off32[AM == A_STAGED ? FM : 1][4];  // byte offsets from g.a (the host checks M * K * 2 < 4 GB)
   const int64_t a_row_bytes = AM == A_NIBBLE ? g.K / 2 : g.K;
   const int64_t w_row_bytes = g.K * BITS / 8;
+  // (row index and row length fit 32 bits - the launcher checks the sizes - so a row's byte offset is one
+  // 32 x 32 -> 64 bit multiply instead of the four quarter-rate multiplies of a 64-bit product)
+  const int m_base32 = pid_m * TM + wm, n_base32 = pid_n * TN + wn;
+  const uint32_t a_row_bytes32 = static_cast<uint32_t>(AM == A_NIBBLE ? K32 / 2 : K32);
+  const uint32_t w_row_bytes32 = static_cast<uint32_t>(K32) * BITS / 8;
+  auto row_offset = [](int row, uint32_t row_bytes) {
+    return static_cast<uint64_t>(static_cast<uint32_t>(row)) * static_cast<uint64_t>(row_bytes);
+  };
   const uint8_t *ap[FM];
   const uint8_t *wp[FN];
 #pragma unroll
@@ -199,10 +214,10 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
       for (int v = 0; v < 4; ++v)
         a_off32[i][v] = static_cast<uint32_t>(min(m_base + 32 * i + 8 * v + (lane >> 3), g.M - 1) * (g.K * 2) + (lane & 7) * 16);
     } else if constexpr (AM == A_TILED) ap[i] = g.a + min(m_base / 32 + i, (g.M + 31) / 32 - 1) * (g.K / 64) * kAStep + lane * 16;
-    else ap[i] = g.a + min(m_base + 32 * i + r, g.M - 1) * a_row_bytes + grp * (kAStep / 2);
+    else ap[i] = g.a + row_offset(min(m_base32 + 32 * i + r, M32 - 1), a_row_bytes32) + grp * (kAStep / 2);
   }
 #pragma unroll
-  for (int j = 0; j < FN; ++j) wp[j] = g.w + min(n_base + 32 * j + r, g.N - 1) * w_row_bytes + grp * (4 * BITS);
+  for (int j = 0; j < FN; ++j) wp[j] = g.w + row_offset(min(n_base32 + 32 * j + r, N32 - 1), w_row_bytes32) + grp * (4 * BITS);
 
   // packed operands of NBUF consecutive K-steps
   uint4 pa[NBUF][FM][kAVec];
@@ -242,9 +257,20 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
 #pragma unroll
     for (int e = 0; e < FM + FN; ++e) fetch_one(buf, e, ks);
   };
+#ifdef OQ_GEMM_STAMPS
+  __asm__ volatile("" ::"v"(wp[FN - 1]), "v"(ap[FM - 1]));
+  __builtin_amdgcn_sched_barrier(0);
+  stamp_extra[4] = __builtin_amdgcn_s_memtime();  // operand addresses computed
+  __builtin_amdgcn_sched_barrier(0);
+#endif
   // buffers 0..NBUF-2 <- K-steps 0..NBUF-2; K-step NBUF-1 is requested by the first step of the loop
   fetch(std::integral_constant<int, 0>{}, 0);
   if constexpr (NBUF == 3) fetch(std::integral_constant<int, 1>{}, 1);
+#ifdef OQ_GEMM_STAMPS
+  __builtin_amdgcn_sched_barrier(0);
+  stamp_extra[5] = __builtin_amdgcn_s_memtime();  // first packed operands requested
+  __builtin_amdgcn_sched_barrier(0);
+#endif
 
   // behind the operands (a wavefront's loads return in order): what only the epilogue needs
   // The window of an output map (an activation function as a table, gemm_epilogue.h) is requested with
@@ -565,7 +591,7 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
     __asm__ volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
     dst[9] = (static_cast<uint64_t>(xcc) << 32) | hw;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dst[10 + i] = stamp_extra[i];
+    for (int i = 0; i < 6; ++i) dst[10 + i] = stamp_extra[i];
   }
 #endif
 #undef OQ_STAMP
@@ -584,7 +610,7 @@ int launch_cfg(GemmArgs g, hipStream_t stream) {
   // a mapped launch parks the map's window in LDS ahead of its main loop (not for partial tiles: they are not mapped)
   g.window_ahead = (g.out_map.table != nullptr && g.out_map.lo == kWideLoBf16 && g.out_dtype == OQ_BF16 && splits == 1 &&
                     reserve_dynamic_lds(reinterpret_cast<const void *>(kern), kWideBytes)) ? 1 : 0;
-  if (g.M > 0x7fffffffLL || g.N > 0x7fffffffLL || g.K > 0x7fffffffLL || g.a_levels > 0xffff)
+  if (g.M > 0x7fff0000LL || g.N > 0x7fff0000LL || g.K > 0x0fffffffLL || g.a_levels > 0xffff)  // (the kernel's 32-bit row and byte counts)
     return fail(OQ_ERR_UNSUPPORTED, "packed_gemm: a dimension beyond 2^31");
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(total), splits), dim3(256), g.window_ahead ? kWideBytes : 0, stream,
                      g.w_cents, g.act_cents, g.a, g.w, g.out_map.table, static_cast<int>(g.K), static_cast<int>(g.M),
