@@ -343,7 +343,7 @@ class RawLinear:
                               (x.data_ptr(), dt, m, k, *rot, levels, *consts, ops._ptr(plan), *q_tail))
         else:
             self._quantize = (self.lib.oq_rotate_quantize_mapped,
-                              (x.data_ptr(), dt, imap.data_ptr(), m, k, *rot, levels, *consts, *q_tail))
+                              (x.data_ptr(), dt, imap.data_ptr(), m, k, *rot, levels, *consts, ops._ptr(plan), *q_tail))
         bias = layer.bias
         g_args = (self.codes.data_ptr(), fmt, self.norms.data_ptr(), layer._activation_codebook_centroids.data_ptr(),
                   int(layer.activation_bits), packed.data_ptr(), int(w_bits), layer.row_norms.data_ptr(), w_cents.data_ptr(),

@@ -137,7 +137,8 @@ int oq_quantize_weight(const void *w, int w_dtype, int64_t N, int64_t K, const v
  * input given as a table: input_map[bits of x] = bits of f(x), 65536 entries of
  * the same dtype as x, 16-byte aligned, on the device.  The result is what
  * oq_rotate_quantize returns for the tensor f(x), bit for bit; f(x) is never
- * written to memory.  x_dtype must be OQ_F16 or OQ_BF16.
+ * written to memory.  x_dtype must be OQ_F16 or OQ_BF16.  rotate_plan: as for
+ * oq_rotate_quantize (bf16 rows into codes take the plan-based kernel with it).
  *
  * No counterpart in the reference's extension: there the activation between two
  * quantized linears (the GELU of an MLP, functional calls in the model code) is
@@ -150,7 +151,7 @@ int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_
                               int64_t M, int64_t K,
                               const int32_t *perm, const int8_t *signs,
                               const float *boundaries, const float *centroids, int levels,
-                              int64_t block, float eps, float inv_sqrt_block,
+                              int64_t block, float eps, float inv_sqrt_block, const void *rotate_plan,
                               void *codes_out, int code_format,
                               void *values_out, int values_mode,
                               float *norms_out, void *stream);

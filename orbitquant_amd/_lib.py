@@ -55,7 +55,7 @@ def load() -> ctypes.CDLL:
     lib.oq_quantize_weight.restype = c_int
     lib.oq_quantize_weight.argtypes = [vp, c_int, c_i64, c_i64, vp, vp, c_int, c_i64, c_f, c_f, c_int, vp, vp, vp]
     lib.oq_rotate_quantize_mapped.restype = c_int
-    lib.oq_rotate_quantize_mapped.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f,
+    lib.oq_rotate_quantize_mapped.argtypes = [vp, c_int, vp, c_i64, c_i64, vp, vp, vp, vp, c_int, c_i64, c_f, c_f, vp,
                                               vp, c_int, vp, c_int, vp, vp]
     lib.oq_debug_override.restype = c_int
     lib.oq_debug_override.argtypes = [ctypes.c_char_p, ctypes.c_char_p]

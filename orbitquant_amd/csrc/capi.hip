@@ -228,12 +228,12 @@ int oq_rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *
 int oq_rotate_quantize_mapped(const void *x, int x_dtype, const uint16_t *input_map, int64_t M, int64_t K,
                               const int32_t *perm, const int8_t *signs, const float *boundaries,
                               const float *centroids, int levels, int64_t block, float eps, float inv_sqrt_block,
-                              void *codes_out, int code_format, void *values_out, int values_mode,
-                              float *norms_out, void *stream) {
+                              const void *rotate_plan, void *codes_out, int code_format, void *values_out,
+                              int values_mode, float *norms_out, void *stream) {
   if (input_map == nullptr) return fail(OQ_ERR_INVALID, "rotate_quantize_mapped: input_map is null");
   return rotate_quantize_dispatch(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
                                   inv_sqrt_block, codes_out, code_format, values_out, values_mode, norms_out,
-                                  input_map, nullptr, as_stream(stream));
+                                  input_map, rotate_plan, as_stream(stream));
 }
 
 int oq_quantize_weight(const void *w, int w_dtype, int64_t N, int64_t K, const void *rotate_plan,

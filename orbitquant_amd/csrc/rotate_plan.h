@@ -62,7 +62,7 @@ int rotate_plan_build(const int32_t *perm, const int8_t *signs, const float *bou
 // -1: this plan / shape has no fast kernel (the caller takes the plain one); else a status.
 int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const void *plan, int levels, int64_t block,
                          float eps, const float *centroids, void *codes_out, int code_format, void *values_out,
-                         int values_mode, float *norms_out, hipStream_t stream);
+                         int values_mode, float *norms_out, const uint16_t *input_map, hipStream_t stream);
 
 // The weight side of a layer on the GPU (rotate_quantize_fast.hip): packed index stream + bf16 row norms.
 int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const void *plan, const float *boundaries,

@@ -132,7 +132,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                              void *codes_out, int code_format, void *values_out, int values_mode,
                              float *norms_out, const uint16_t *input_map, const void *plan, hipStream_t stream) {
   // With a rotate plan, launches of more than a few rows take the plan-based kernel (same results);
-  // decode-sized launches and fused input maps stay with the kernel below, which is built for latency.
+  // decode-sized launches (and input maps on anything but bf16 rows into codes) stay with the kernel below, which is built for latency.
   // The plan kernel gives every 512-slot unit (or block, if larger) of a row to one wavefront.  With many rows that is
   // all the parallelism it needs; with at most sixteen rows it wins only when a row has several units (K = 14336
   // in blocks of 2048, one token: 7.9 us against 10.1 us; K = 1152: 3.8 against 4.4) and loses when the row is one
@@ -146,7 +146,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
   const bool several_units = (K + unit - 1) / unit >= 3;
   if (block >= 2048 && !several_units) fast_min_m = 513;
   if (const char *v = debug_env(ENV_RQ_FAST_MIN_M)) fast_min_m = atoi(v);
-  if (plan != nullptr && input_map == nullptr && (M >= fast_min_m || several_units)) {
+  if (plan != nullptr && (input_map == nullptr || x_dtype == OQ_BF16) && (M >= fast_min_m || several_units)) {
     RqArgs checked;
     bool vec_checked = false;
     if (int rc = rotate_quantize_prepare(x, x_dtype, M, K, perm, signs, boundaries, centroids, levels, block, eps,
@@ -154,7 +154,7 @@ int rotate_quantize_dispatch(const void *x, int x_dtype, int64_t M, int64_t K, c
                                          input_map, &checked, &vec_checked))
       return rc;
     const int rc = rotate_quantize_fast(x, x_dtype, M, K, plan, levels, block, eps, centroids, codes_out, code_format,
-                                        values_out, values_mode, norms_out, stream);
+                                        values_out, values_mode, norms_out, input_map, stream);
     if (rc >= 0) return rc;
   }
   RqArgs a;

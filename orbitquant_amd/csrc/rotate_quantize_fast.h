@@ -28,6 +28,7 @@
 #include "packed_decode.h"
 #include "rotate_plan.h"
 #include "rotate_quantize_row.h"
+#include "value_map.h"
 
 namespace oq {
 namespace rqf {
@@ -58,13 +59,18 @@ struct FastArgs {
   int pack_bits;
   uint8_t *packed;           // flat bit stream of [M, K] indices
   uint16_t *norms_bf16;      // [M]
+  // MAPPED only: a function of the 16-bit input as a table of 65536 entries (value_map.h), applied to
+  // every value as it is read; what follows - norm, rotation, codes - is that of the mapped row
+  const uint16_t *map;
 };
 
 // LDS: cells (2048) | thresholds (1024) | centroids (1024) | reduction slots (64) | staging
 constexpr int kCellsAt = 0, kThrAt = 2048, kCentAt = 3072, kRedAt = 4096, kStageAt = plan::kStageAddress;  // kRedAt: four group sums, then one flag per wavefront
 
 // staging: 4 bytes per value (fp32 once, 16-bit twice)
-inline size_t fast_lds_bytes(int64_t K) { return static_cast<size_t>(kStageAt) + 4u * static_cast<size_t>(K); }
+__host__ __device__ inline size_t fast_lds_bytes(int64_t K) { return static_cast<size_t>(kStageAt) + 4u * static_cast<size_t>(K); }
+// ... and behind it, for a launch with an input map, the map's 16 KB window (value_map.h)
+inline size_t fast_lds_bytes_mapped(int64_t K) { return fast_lds_bytes(K) + static_cast<size_t>(kWideBytes); }
 
 // ---- lane-exchange butterflies, eight values per call -------------------------------------------
 // y'[lane] = (lane & J) ? y[lane ^ J] - y[lane] : y[lane] + y[lane ^ J]
@@ -182,9 +188,10 @@ enum EmitMode { EMIT_NIBBLE = 0, EMIT_U8 = 1, EMIT_ANY = 2, EMIT_WEIGHT = 3 };
 
 // One row.  `smem`: fast_lds_bytes(K) bytes, 16-byte aligned.  All 64 * waves threads of the
 // workgroup make the call.
-template <int DT, int LOG_H, int EMIT>
+template <int DT, int LOG_H, int EMIT, bool MAPPED = false>
 __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsigned char *smem, const int64_t row,
                                                          const int tid, const int waves) {
+  static_assert(!MAPPED || DT == OQ_BF16, "the input map's LDS window is one of bf16 bit patterns");
   constexpr int H = 1 << LOG_H;
   constexpr int G = H > kLaneSpan ? H / kLaneSpan : 1;  // steps of 512 values a unit is made of
   const int lane = tid & 63, wave = tid >> 6;
@@ -219,6 +226,15 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
   const float thr_v = EMIT == EMIT_WEIGHT ? (table_idx < a.levels - 1 ? a.raw_bounds[table_idx] : __builtin_inff())
                                           : reinterpret_cast<const float *>(a.plan + plan::kThresholdsOffset)[table_idx];
   const float cent_v = (EMIT == EMIT_ANY && a.cents != nullptr) ? a.cents[min(table_idx, a.levels - 1)] : 0.0f;
+
+  // an input map's window goes to LDS first (every wavefront looks values up in it as it reads the row)
+  const uint16_t *hot = nullptr;
+  if constexpr (MAPPED) {
+    uint16_t *window = reinterpret_cast<uint16_t *>(smem + fast_lds_bytes(K));
+    fill_map_window<kWideLog2>(window, a.map, kWideLoBf16, tid, waves * 64);
+    hot = window;
+    __syncthreads();
+  }
 
   // ---- phase A: stage the row (16-bit inputs as x and as -x), sum of squares -----------------
   // Virtual lane t of the documented [passes][256 lanes][8] order is lane t % 64 of group t / 64;
@@ -270,9 +286,18 @@ __device__ __forceinline__ void rotate_quantize_row_fast(const FastArgs &a, unsi
               tiny32 = tiny32 || (f[e] != 0.0f && __builtin_fabsf(f[e]) < 0x1p-80f);
             }
           } else {
-            const uint32_t w[4] = {raw_lo[b].x, raw_lo[b].y, raw_lo[b].z, raw_lo[b].w};
+            uint4 in = raw_lo[b];
+            if constexpr (MAPPED) {
+              // (lanes past the row's end look up an ordinary value instead of their zero padding, which lies
+              // outside the window and would send the whole wavefront to the table in memory; they add +0 as before)
+              const bool live = i0 < Ki;
+              uint4 one[1] = {live ? in : make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u)};
+              map_words8_many<OQ_BF16, 1, kWideLog2>(one, a.map, hot, kWideLoBf16);
+              in = live ? one[0] : make_uint4(0u, 0u, 0u, 0u);
+            }
+            const uint32_t w[4] = {in.x, in.y, in.z, in.w};
             if (i0 < Ki) {
-              *reinterpret_cast<uint4 *>(stage + 2 * i0) = raw_lo[b];
+              *reinterpret_cast<uint4 *>(stage + 2 * i0) = in;
               *reinterpret_cast<uint4 *>(stage + 2 * (Ki + i0)) =
                   make_uint4(w[0] ^ 0x80008000u, w[1] ^ 0x80008000u, w[2] ^ 0x80008000u, w[3] ^ 0x80008000u);
             }

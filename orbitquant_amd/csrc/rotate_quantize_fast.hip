@@ -95,15 +95,15 @@ __global__ __launch_bounds__(256) void rotate_plan_build_kernel(const int32_t *p
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
-template <int DT, int LOG_H, int EMIT>
+template <int DT, int LOG_H, int EMIT, bool MAPPED>
 __global__ __launch_bounds__(512) void rotate_quantize_fast_kernel(FastArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  rotate_quantize_row_fast<DT, LOG_H, EMIT>(a, smem, blockIdx.x, threadIdx.x, blockDim.x >> 6);
+  rotate_quantize_row_fast<DT, LOG_H, EMIT, MAPPED>(a, smem, blockIdx.x, threadIdx.x, blockDim.x >> 6);
 }
 
-template <int DT, int LOG_H, int EMIT>
+template <int DT, int LOG_H, int EMIT, bool MAPPED = false>
 int launch_emit(const FastArgs &a, int waves, size_t smem, hipStream_t stream) {
-  auto kern = rotate_quantize_fast_kernel<DT, LOG_H, EMIT>;
+  auto kern = rotate_quantize_fast_kernel<DT, LOG_H, EMIT, MAPPED>;
   if (!reserve_dynamic_lds(reinterpret_cast<const void *>(kern), smem))
     return fail(OQ_ERR_LAUNCH, "rotate_quantize: cannot reserve %zu bytes of LDS", smem);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(a.M)), dim3(64 * waves), smem, stream, a);
@@ -112,6 +112,15 @@ int launch_emit(const FastArgs &a, int waves, size_t smem, hipStream_t stream) {
 
 template <int DT, int LOG_H>
 int launch_one(const FastArgs &a, int waves, size_t smem, hipStream_t stream) {
+  if (a.map != nullptr) {  // an input map: bf16 rows into codes only (the forms the layers use); -1 sends the rest to the plain kernel
+    if constexpr (DT == OQ_BF16) {
+      if (a.packed == nullptr && a.codes != nullptr && a.values == nullptr) {
+        if (a.code_format == OQ_CODES_NIBBLE) return launch_emit<DT, LOG_H, EMIT_NIBBLE, true>(a, waves, smem, stream);
+        return launch_emit<DT, LOG_H, EMIT_U8, true>(a, waves, smem, stream);
+      }
+    }
+    return -1;
+  }
   if (a.packed != nullptr) return launch_emit<DT, LOG_H, EMIT_WEIGHT>(a, waves, smem, stream);
   if (a.codes != nullptr && a.values == nullptr) {
     if (a.code_format == OQ_CODES_NIBBLE) return launch_emit<DT, LOG_H, EMIT_NIBBLE>(a, waves, smem, stream);
@@ -184,7 +193,7 @@ int quantize_weight_fast(const void *w, int w_dtype, int64_t N, int64_t K, const
 
 int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const void *plan, int levels, int64_t block,
                          float eps, const float *centroids, void *codes_out, int code_format, void *values_out,
-                         int values_mode, float *norms_out, hipStream_t stream) {
+                         int values_mode, float *norms_out, const uint16_t *input_map, hipStream_t stream) {
   auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   int log_h = 0;
   while ((int64_t{1} << log_h) < block) ++log_h;
@@ -200,6 +209,7 @@ int rotate_quantize_fast(const void *x, int x_dtype, int64_t M, int64_t K, const
   a.codes = static_cast<uint8_t *>(codes_out); a.code_format = code_format;
   a.values = values_mode == OQ_VALUES_NONE ? nullptr : values_out; a.values_mode = values_mode;
   a.norms = norms_out;
+  a.map = input_map;
   return launch_fast(a, x_dtype, stream);
 }
 
@@ -222,7 +232,7 @@ static int launch_fast(FastArgs &a, int x_dtype, hipStream_t stream) {
     const int w = atoi(forced);
     if (w >= 1 && w <= 8) waves = w < a.units ? w : a.units;
   }
-  const size_t smem = fast_lds_bytes(K);
+  const size_t smem = a.map != nullptr ? fast_lds_bytes_mapped(K) : fast_lds_bytes(K);
   if (smem > 160 * 1024) return -1;
   switch (x_dtype) {
     case OQ_F32: return launch_dtype<OQ_F32>(a, log_h, waves, smem, stream);

@@ -232,7 +232,7 @@ def rotate_quantize(
         if input_map is None:
             rc = lib.oq_rotate_quantize(rows.data_ptr(), _dt(rows), *head, _ptr(plan), *tail)
         else:
-            rc = lib.oq_rotate_quantize_mapped(rows.data_ptr(), _dt(rows), input_map.data_ptr(), *head, *tail)
+            rc = lib.oq_rotate_quantize_mapped(rows.data_ptr(), _dt(rows), input_map.data_ptr(), *head, _ptr(plan), *tail)
     _lib.check(rc, "oq_rotate_quantize")
     if codes is not None:
         codes = codes.reshape(*lead, codes.shape[-1])

@@ -88,6 +88,40 @@ def test_mapped_quantizer_equals_quantizer_of_mapped_tensor(dev, m, k, abits, dt
             assert torch.equal(a, b), f"{name} differ"
 
 
+PLAN_MAP_CASES = [
+    # m, k, abits, code_format, fn, scale, block: bf16 rows into codes, the forms the plan-based kernel takes with a map
+    (2048, 4608, 4, "nibble", gelu, 1.6, "paper"),     # the MLP pair's second quantizer (three passes, nine units)
+    (300, 1152, 4, "nibble", gelu, 1.0, "paper"),      # lanes past the row's end in the last pass
+    (64, 4608, 4, "u8", gelu, 1e-3, "paper"),          # most values below the window: the table in memory
+    (33, 12288, 3, "nibble", gelu_tanh, 40.0, "paper"),  # block 4096, saturated values
+    (100, 3072, 6, "u8", torch.nn.functional.silu, 1.0, 64),
+    (17, 2048, 4, "nibble", torch.relu, 1.0, 8),       # the smallest block; half the mapped values are zero
+]
+
+
+@pytest.mark.parametrize(("m", "k", "abits", "fmt", "fn", "scale", "block"), PLAN_MAP_CASES)
+def test_mapped_plan_kernel_equals_plan_kernel_on_the_mapped_tensor(dev, m, k, abits, fmt, fn, scale, block):
+    """With a rotate plan the mapped quantizer runs the plan-based kernel (the table's window in LDS, every
+    value looked up as the row is read); its codes and norms are those of the same kernel on f(x), and of
+    the plain kernel through the map, bit for bit."""
+    from orbitquant_amd import ops
+
+    c = rotation_and_tables(k, abits, dev, block)
+    x = make_input(m, k, torch.bfloat16, scale, seed=3 * m + k).to(dev)
+    table = ops.activation_table(fn, torch.bfloat16, dev)
+    levels = c["bounds"].numel() + 1
+    plan = ops.rotate_plan(c["perm"], c["signs"], c["bounds"], block_size=c["block"], inv_sqrt_block=float(c["inv"]))
+    kw = dict(block_size=c["block"], eps=1e-10, inv_sqrt_block=float(c["inv"]), code_format=fmt)
+    want = ops.rotate_quantize(fn(x), c["perm"], c["signs"], c["bounds"], plan=plan, **kw)
+    plain = ops.rotate_quantize(x, c["perm"], c["signs"], c["bounds"], input_map=table, **kw)
+    got = ops.rotate_quantize(x, c["perm"], c["signs"], c["bounds"], input_map=table, plan=plan, **kw)
+    assert levels == 1 << abits
+    for name, a, b, p in zip(("codes", "values", "norms"), got, want, plain):
+        if b is not None:
+            assert torch.equal(a, b), f"{name} differ from the plan kernel on f(x)"
+            assert torch.equal(a, p), f"{name} differ from the plain kernel through the map"
+
+
 def test_mapped_quantizer_against_the_oracle(dev):
     from orbitquant_amd import ops
 
@@ -131,7 +165,7 @@ def test_mapped_quantizer_rejects_bad_arguments(dev):
     codes = torch.empty(4, 512, dtype=torch.uint8, device=dev)
     norms = torch.empty(4, device=dev)
     args = (4, 512, c["perm"].data_ptr(), c["signs"].data_ptr(), c["bounds"].data_ptr(), None, 16, c["block"], 1e-10,
-            float(c["inv"]), codes.data_ptr(), 0, None, 0, norms.data_ptr(), None)
+            float(c["inv"]), None, codes.data_ptr(), 0, None, 0, norms.data_ptr(), None)
     assert lib.oq_rotate_quantize_mapped(x.data_ptr(), 2, None, *args) == 1
     assert lib.oq_rotate_quantize_mapped(x.data_ptr(), 0, table.data_ptr(), *args) == 1
     assert b"16-bit" in lib.oq_last_error()
