@@ -498,7 +498,11 @@ def cpu_baseline(spec, layers, x, target_seconds=15.0):
     run(rows0)
     per_row = (time.perf_counter() - t0) / rows0
     rows = int(min(m, max(rows0, target_seconds / per_row)))
-    reps = max(1, int(round(target_seconds / (per_row * rows)))) if rows == m else 1
+    reps = 1
+    if rows == m:   # whole passes: a pass over all rows runs far better than the 64-row probe predicts, so time one
+        t0 = time.perf_counter()
+        run(rows)
+        reps = max(1, int(round(target_seconds / (time.perf_counter() - t0))))
     t0 = time.perf_counter()
     for _ in range(reps):
         run(rows)
@@ -902,7 +906,7 @@ def gemm_phases(layers, x, launches=20):
         rows = [("start -> kernel arguments read", 0, 10), ("-> centroids requested, tile mapped", 10, 13), ("-> operand addresses", 13, 14), ("-> first packed operands requested", 14, 15),
                 ("-> output-map window requested", 15, 11), ("-> centroids arrived", 11, 12),
                 ("-> lookup tables written", 12, 1), ("-> barrier, first lookups (loop entered)", 1, 2), ("main loop", 2, 3),
-                ("wait at the barrier after the loop", 3, 4), ("epilogue until the last store is issued", 4, 5), ("stores drained", 5, 8)]
+                ("wait at the barrier after the loop", 3, 4), ("epilogue until the last store is issued", 4, 5),  ("stores drained", 5, 8)]
         for name, a, b in rows:
             d = (s[:, b] - s[:, a]).astype(np.float64) / mhz
             print(f"    {name:42s} median {np.median(d):6.2f}   p10 {np.percentile(d, 10):6.2f}   p90 {np.percentile(d, 90):6.2f}   max {d.max():6.2f} us")

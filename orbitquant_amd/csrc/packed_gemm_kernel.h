@@ -514,62 +514,68 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
                           reinterpret_cast<unsigned char *>(lds), out_map, 64 * FM,
                           window_ahead ? reinterpret_cast<const uint16_t *>(map_window) : nullptr);
   } else {
-    // Reduce-scatter over the wavefronts in three rounds: in round d wavefront w hands row slice
-    // (w+d)%4 of its partial tile to wavefront (w+d)%4 and adds what it receives from (w-d)%4 to
-    // its own slice w.  Slot of destination s: [FN tiles][4 runs][64 lanes] of float4.
+    // Reduce-scatter over the wavefronts in four rounds, one per row slice: in round s every wavefront parks
+    // slice s of its partial tile in LDS (slot = its own number) and wavefront s adds the other three to its
+    // own, in the order s-1, s-2, s-3 (mod 4).  The accumulator slices are registers, so which one is sent or
+    // summed has to be a compile-time index: this way it is the round's number, the same instructions for all
+    // four wavefronts (a scheme in which each wavefront sends a different slice per round needs four copies
+    // of every round, each fetched by one wavefront alone, and measured 0.5 us slower a launch).  Every barrier
+    // (and the epilogue, which has one of its own) is reached by all four in the same place.
+    // Slot of wavefront v: [FN tiles][4 runs][64 lanes] of float4.
     float4 *slots = reinterpret_cast<float4 *>(lds);
-    // The accumulator slices are registers, so which one a wavefront sends or keeps has to be a
-    // compile-time index: only the LDS traffic is selected per wavefront, every barrier (and
-    // the epilogue, which has one of its own) is reached by all four in the same place.
-    auto send = [&](auto wt, auto dt) __attribute__((always_inline)) {
-      constexpr int dst = (decltype(wt)::value + decltype(dt)::value) & 3;
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
-        const f32x16 t = acc[dst][j];  // whole-tile copies keep the accumulators in registers
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4)
-          slots[((dst * FN + j) * 4 + a4) * 64 + lane] = make_float4(t[4 * a4 + 0], t[4 * a4 + 1], t[4 * a4 + 2], t[4 * a4 + 3]);
-      }
-    };
-    // the last round's sum is the wavefront's own slice of the finished tile
     f32x16 slice[1][FN];
     EpiFactors<1> mine;
     mine.rn = epi.rn;
     mine.bv = epi.bv;
-    auto receive = [&](auto wt, auto dt) __attribute__((always_inline)) {
-      constexpr int W = decltype(wt)::value;
-      constexpr bool kLast = decltype(dt)::value == 3;
-      if constexpr (kLast) mine.sc[0] = epi.sc[W];
+    mine.sc[0] = 1.0f;
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
-        f32x16 t;
+    for (int j = 0; j < FN; ++j)
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          const float4 v = slots[((W * FN + j) * 4 + a4) * 64 + lane];
-          t[4 * a4 + 0] = v.x;
-          t[4 * a4 + 1] = v.y;
-          t[4 * a4 + 2] = v.z;
-          t[4 * a4 + 3] = v.w;
+      for (int e = 0; e < 16; ++e) slice[0][j][e] = 0.0f;
+    auto round = [&](auto st) __attribute__((always_inline)) {
+      constexpr int S = decltype(st)::value;
+      if (wave != S) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const f32x16 t = acc[S][j];  // whole-tile copies keep the accumulators in registers
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4)
+            slots[((wave * FN + j) * 4 + a4) * 64 + lane] = make_float4(t[4 * a4 + 0], t[4 * a4 + 1], t[4 * a4 + 2], t[4 * a4 + 3]);
         }
-        if constexpr (kLast) slice[0][j] = acc[W][j] + t;
-        else acc[W][j] += t;
       }
+      __syncthreads();
+      if (wave == S) {
+        mine.sc[0] = epi.sc[S];
+        // the twelve reads of a tile are issued before its first sum (one LDS round trip a tile, not one a read)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          float4 part[3][4];
+#pragma unroll
+          for (int d = 1; d < 4; ++d)
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4)
+              part[d - 1][a4] = slots[((((S + 4 - d) & 3) * FN + j) * 4 + a4) * 64 + lane];
+          __builtin_amdgcn_sched_barrier(0);
+          f32x16 sum = acc[S][j];
+#pragma unroll
+          for (int d = 0; d < 3; ++d)
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+              sum[4 * a4 + 0] += part[d][a4].x;
+              sum[4 * a4 + 1] += part[d][a4].y;
+              sum[4 * a4 + 2] += part[d][a4].z;
+              sum[4 * a4 + 3] += part[d][a4].w;
+            }
+          slice[0][j] = sum;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (S < 3) __syncthreads();  // the slots are written again by the next round
     };
-#define OQ_KSPLIT_ROUND(D)                                                              \
-    if (wave == 0) send(std::integral_constant<int, 0>{}, std::integral_constant<int, D>{});      \
-    else if (wave == 1) send(std::integral_constant<int, 1>{}, std::integral_constant<int, D>{}); \
-    else if (wave == 2) send(std::integral_constant<int, 2>{}, std::integral_constant<int, D>{}); \
-    else send(std::integral_constant<int, 3>{}, std::integral_constant<int, D>{});                \
-    __syncthreads();                                                                    \
-    if (wave == 0) receive(std::integral_constant<int, 0>{}, std::integral_constant<int, D>{});      \
-    else if (wave == 1) receive(std::integral_constant<int, 1>{}, std::integral_constant<int, D>{}); \
-    else if (wave == 2) receive(std::integral_constant<int, 2>{}, std::integral_constant<int, D>{}); \
-    else receive(std::integral_constant<int, 3>{}, std::integral_constant<int, D>{});                \
-    __syncthreads();
-    OQ_KSPLIT_ROUND(1)
-    OQ_KSPLIT_ROUND(2)
-    OQ_KSPLIT_ROUND(3)
-#undef OQ_KSPLIT_ROUND
+    round(std::integral_constant<int, 0>{});
+    round(std::integral_constant<int, 1>{});
+    round(std::integral_constant<int, 2>{});
+    round(std::integral_constant<int, 3>{});
     gemm_epilogue<1, FN>(slice, static_cast<int64_t>(pid_m) * TM, static_cast<int64_t>(pid_n) * TN, 32 * wave, 0, TN, tid, g.M,
                          g.N, g.row_scale, g.row_norms, g.bias, g.bias_dtype, mine, g.out, g.out_dtype,
                          reinterpret_cast<unsigned char *>(lds), g.out_map, TM,
