@@ -280,14 +280,13 @@ __global__ __launch_bounds__(256) void packed_gemm_kernel(const float *w_cents, 
   const bool window_ahead = g.window_ahead != 0;  // uniform
   // (requested without a branch - a launch without a map reads the first bytes of the weights - and held as
   // native vectors: an array of the struct type would be pinned in scratch memory)
-  lds_u32x4 window_piece0, window_piece1, window_piece2, window_piece3;
-  {
+  lds_u32x4 window_piece0, window_piece1, window_piece2, window_piece3;  // written and read under the same uniform condition only
+  if (window_ahead) {
     constexpr int kChunksPerSign = (2 << kWideLog2) / 16;
-    const unsigned char *window_from = window_ahead ? reinterpret_cast<const unsigned char *>(g.out_map.table + kWideLoBf16)  // (the launcher parks windows of this base only)
-                                                    : reinterpret_cast<const unsigned char *>(g.w);
+    const unsigned char *window_from = reinterpret_cast<const unsigned char *>(g.out_map.table + kWideLoBf16);  // (the launcher parks windows of this base only)
     auto piece = [&](int v) {
       const int i = tid + 256 * v, sign = i / kChunksPerSign, j = i % kChunksPerSign;
-      return *reinterpret_cast<const lds_u32x4 *>(window_from + (window_ahead ? (sign << 16) + 16 * j : 0));
+      return *reinterpret_cast<const lds_u32x4 *>(window_from + (sign << 16) + 16 * j);
     };
     window_piece0 = piece(0);
     window_piece1 = piece(1);
